@@ -9,7 +9,7 @@ loading is supported for real weights.
 from __future__ import annotations
 
 import dataclasses
-from typing import Optional
+from typing import List, Optional
 
 
 @dataclasses.dataclass
@@ -32,6 +32,8 @@ class ModelSpec:
     moe_intermediate_size: Optional[int] = None
     moe_shared_experts: int = 0
     moe_dtype: str = "bf16"  # "fp8" enables the CDNA4 fp8 expert GEMM path
+
+    is_hybrid = False
 
     @property
     def is_moe(self) -> bool:
@@ -169,7 +171,208 @@ MODEL_REGISTRY = {
 }
 
 
-def get_model_spec(name: str) -> ModelSpec:
+def get_model_spec(name):
+    """A registry name, a checkpoint folder, or an already-built spec."""
+    import os
+
+    if not isinstance(name, str):
+        return name
+    if name in HYBRID_REGISTRY:
+        return povazen_spec_from_dict(HYBRID_REGISTRY[name](), name=name)
+    if os.path.isdir(name) and os.path.exists(os.path.join(name, "config.json")):
+        return load_spec_from_dir(name)
     if name not in MODEL_REGISTRY:
         raise KeyError(f"unknown model {name!r}; known: {sorted(MODEL_REGISTRY)}")
     return MODEL_REGISTRY[name]
+
+
+# ---------------------------------------------------------------------------
+# Hybrid designs: a per-layer list of mixers (softmax attention, recurrent
+# delta rule, ...) read from a checkpoint folder's config.json. Every size
+# and every constant that can differ between checkpoints lives in the spec;
+# nothing is taken from a particular checkpoint.
+
+
+@dataclasses.dataclass
+class MixerSpec:
+    """One layer's token mixer. kind: "attention" | "channel_delta"."""
+
+    kind: str
+    heads: int
+    kv_heads: int
+    dim: int                      # per-head query/key size
+    vdim: int                     # per-head value size
+    scale: Optional[float] = None  # attention score scale
+    conv: int = 0                 # short-convolution taps (recurrent mixers)
+    # inner sizes of the low-rank decay / output-gate projections; only the
+    # checkpoint's tensor shapes give them (None => the mixer's default)
+    decay_rank: Optional[int] = None
+    gate_rank: Optional[int] = None
+
+    @property
+    def has_kv(self) -> bool:
+        return self.kind == "attention"
+
+    @property
+    def has_state(self) -> bool:
+        return self.kind == "channel_delta"
+
+
+@dataclasses.dataclass
+class HybridLayerSpec:
+    mixer: MixerSpec
+    mlp_kind: Optional[str] = None   # None => the layer has no feed-forward
+    mlp_ff: int = 0
+
+
+@dataclasses.dataclass
+class HybridSpec:
+    """Architecture of a hybrid decoder (the Povazen design)."""
+
+    name: str
+    architecture: str
+    vocab_size: int
+    hidden_size: int
+    layers: List[HybridLayerSpec]
+    norm_eps: float
+    norm_groups: int
+    canon_taps: int
+    logit_softcap: float
+    max_seq_len: int = 1 << 20
+    weights_path: Optional[str] = None
+
+    is_moe = False
+    is_hybrid = True
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+
+def povazen_spec_from_dict(cfg: dict, name: str = "povazen") -> HybridSpec:
+    """Parse a Povazen config.json dict."""
+    layers = []
+    for entry in cfg["layers"]:
+        m = entry["mixer"]
+        kind = entry["type"]
+        if kind not in ("attention", "channel_delta"):
+            raise ValueError(f"unknown Povazen layer type {kind!r}")
+        mixer = MixerSpec(
+            kind=kind,
+            heads=int(m["heads"]),
+            kv_heads=int(m["kv_heads"]),
+            dim=int(m["dim"]),
+            vdim=int(m["vdim"]),
+            scale=float(m["scale"]) if "scale" in m else None,
+            conv=int(m.get("conv", 0)),
+        )
+        if mixer.heads % mixer.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        mlp = entry.get("mlp")
+        if mlp is not None and mlp.get("kind") != "dense":
+            raise ValueError(f"unknown Povazen feed-forward kind {mlp.get('kind')!r}")
+        layers.append(
+            HybridLayerSpec(
+                mixer=mixer,
+                mlp_kind=None if mlp is None else "dense",
+                mlp_ff=0 if mlp is None else int(mlp["ff"]),
+            )
+        )
+    width = int(cfg["width"])
+    groups = int(cfg["norm"]["groups"])
+    if width % groups:
+        raise ValueError("width must be a multiple of norm.groups")
+    return HybridSpec(
+        name=name,
+        architecture="Povazen",
+        vocab_size=int(cfg["vocab"]),
+        hidden_size=width,
+        layers=layers,
+        norm_eps=float(cfg["norm"]["eps"]),
+        norm_groups=groups,
+        canon_taps=int(cfg["canon"]["taps"]),
+        logit_softcap=float(cfg["logit_softcap"]),
+    )
+
+
+def povazen_config_dict(
+    vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int,
+    vdim: int, ff: int, delta_heads: Optional[int] = None, conv: int = 4,
+    taps: int = 3, groups: int = 4, eps: float = 1e-6, softcap: float = 30.0,
+) -> dict:
+    """A Povazen config.json dict from a layer pattern: 'D' = channel_delta
+    layer without feed-forward, 'd' = with one, 'A'/'a' likewise attention."""
+    layers = []
+    for ch in pattern:
+        mlp = {"kind": "dense", "ff": ff} if ch.islower() else None
+        if ch in "Aa":
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim,
+                     "vdim": vdim, "scale": dim ** -0.5}
+            layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+        else:
+            dh = delta_heads or heads
+            mixer = {"heads": dh, "kv_heads": dh, "dim": dim, "vdim": vdim, "conv": conv}
+            layers.append({"type": "channel_delta", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Povazen", "canon": {"taps": taps}, "layers": layers,
+            "logit_softcap": softcap, "norm": {"eps": eps, "groups": groups},
+            "vocab": vocab, "width": width}
+
+
+# config.json "architecture" -> parser
+ARCHITECTURE_PARSERS = {"Povazen": povazen_spec_from_dict}
+
+# named hybrid configurations (random-weight benchmarking and tests)
+HYBRID_REGISTRY = {
+    # CPU-test size
+    "povazen-tiny": lambda: povazen_config_dict(
+        vocab=512, width=64, pattern="Dad", heads=4, kv_heads=2, dim=16, vdim=8,
+        ff=128, delta_heads=2),
+    # GPU-smoke size
+    "povazen-micro": lambda: povazen_config_dict(
+        vocab=2048, width=1024, pattern="DdaD", heads=8, kv_heads=2, dim=128,
+        vdim=128, ff=2816, delta_heads=8),
+    # layer shapes of an ~8B-class model at 4 layers (speed measurements
+    # beside llama3 layers of equal width)
+    "povazen-4l4k": lambda: povazen_config_dict(
+        vocab=2048, width=4096, pattern="dada", heads=32, kv_heads=8, dim=128,
+        vdim=128, ff=14336, delta_heads=32),
+}
+
+
+def load_spec_from_dir(path: str):
+    """Model spec from a checkpoint folder (config.json + model.safetensors);
+    the model class follows config.json's "architecture"."""
+    import json
+    import os
+
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    arch = cfg.get("architecture")
+    if arch not in ARCHITECTURE_PARSERS:
+        raise KeyError(
+            f"unknown architecture {arch!r} in {path}/config.json; "
+            f"known: {sorted(ARCHITECTURE_PARSERS)}"
+        )
+    spec = ARCHITECTURE_PARSERS[arch](cfg, name=os.path.basename(os.path.normpath(path)))
+    spec.weights_path = os.path.join(path, "model.safetensors")
+    if os.path.exists(spec.weights_path):
+        shapes = safetensors_shapes(spec.weights_path)
+        for i, layer in enumerate(spec.layers):
+            a1, g1 = shapes.get(f"l{i}.mix.a1"), shapes.get(f"l{i}.mix.g1")
+            if a1 is not None:
+                layer.mixer.decay_rank = int(a1[0])
+            if g1 is not None:
+                layer.mixer.gate_rank = int(g1[0])
+    return spec
+
+
+def safetensors_shapes(path: str) -> dict:
+    """name -> shape from a safetensors header (8-byte little-endian length,
+    then that many bytes of JSON); reads no tensor data."""
+    import json
+    import struct
+
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(n))
+    return {k: tuple(v["shape"]) for k, v in header.items() if k != "__metadata__"}

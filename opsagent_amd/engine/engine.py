@@ -35,6 +35,7 @@ from opsagent_amd.engine.kv_cache import (
     BlockAllocatorError,
     PagedKVCache,
     SequenceState,
+    StateSlotPool,
 )
 from opsagent_amd.engine.model import ForwardBatch, LlamaForCausalLM
 from opsagent_amd.engine.tokenizer import ByteTokenizer, get_tokenizer
@@ -130,12 +131,23 @@ _BCAST_MARK = -2
 class LLMEngine:
     def __init__(self, engine_cfg: Optional[dict] = None):
         cfg = dict(engine_cfg or {})
+        # a registry name, or a checkpoint folder (config.json names the
+        # architecture and thereby the model class)
         self.spec: ModelSpec = get_model_spec(cfg.get("model", "llama3-8b"))
+        self.hybrid = bool(getattr(self.spec, "is_hybrid", False))
         if cfg.get("moe_dtype"):
             import dataclasses as _dc
 
             self.spec = _dc.replace(self.spec, moe_dtype=str(cfg["moe_dtype"]))
-        self.dtype = torch.bfloat16 if cfg.get("dtype", "bf16") == "bf16" else torch.float16
+        dtype_name = str(cfg.get("dtype", "bf16")).lower()
+        if dtype_name in ("bf16", "bfloat16"):
+            self.dtype = torch.bfloat16
+        elif dtype_name in ("fp32", "float32"):
+            if not self.hybrid:
+                raise ValueError("float32 serving is implemented for hybrid models only")
+            self.dtype = torch.float32
+        else:
+            self.dtype = torch.float16
         self.max_batch = int(cfg.get("max_batch_size", 64))
         self.block_size = int(cfg.get("kv_block_size", 32))
         self.max_seq_len = min(int(cfg.get("max_seq_len", 8192)), self.spec.max_seq_len)
@@ -209,12 +221,15 @@ class LLMEngine:
         if self.device == "cpu":
             self.use_hipgraph = False
             # keep CPU tests fast/accurate: fp32 reference path
-            self.dtype = torch.float32 if cfg.get("dtype", "bf16") == "bf16" else self.dtype
+            self.dtype = torch.float32 if self.dtype == torch.bfloat16 else self.dtype
 
         self.tokenizer: ByteTokenizer = get_tokenizer(
             cfg.get("tokenizer"), template=str(cfg.get("chat_template", "llama3"))
         )
-        if self.tokenizer.vocab_size > self.spec.vocab_size:
+        # token-id replay needs no tokenizer; text serving does
+        if bool(cfg.get("tokenizer_check", True)) and (
+            self.tokenizer.vocab_size > self.spec.vocab_size
+        ):
             raise ValueError(
                 f"tokenizer vocab ({self.tokenizer.vocab_size}) exceeds the "
                 f"model vocab ({self.spec.vocab_size}) — its token ids would "
@@ -227,9 +242,20 @@ class LLMEngine:
         torch.manual_seed(self.seed)
         log.info("building model %s (tp=%d, dtype=%s, device=%s)",
                  self.spec.name, self.tp, self.dtype, self.device)
-        self.model = LlamaForCausalLM(self.spec, self.dtype, self.device, self.seed)
+        if self.hybrid:
+            from opsagent_amd.engine.hybrid import HybridForCausalLM
+
+            # stateful mixers: no speculative rollback, no key-only prefix reuse
+            self.spec_decode = False
+            self.use_hipgraph = self.use_hipgraph and bool(cfg.get("hybrid_hipgraph", True))
+            self.model = HybridForCausalLM(self.spec, self.dtype, self.device, self.seed)
+        else:
+            self.model = LlamaForCausalLM(self.spec, self.dtype, self.device, self.seed)
         self.model.eval()
-        weights = str(cfg.get("weights", "random") or "random")
+        weights = str(cfg.get("weights", "") or "")
+        if not weights:
+            # a checkpoint folder brings its own weights
+            weights = getattr(self.spec, "weights_path", None) or "random"
         if weights not in ("random", ""):
             from opsagent_amd.engine.loader import load_weights
 
@@ -251,6 +277,31 @@ class LLMEngine:
                 t = t.cuda()
             dist.all_reduce(t, op=dist.ReduceOp.MIN)
             num_blocks = int(t.item())
+        self.state_pool: Optional[StateSlotPool] = None
+        self.requests: Dict[int, Request] = {}
+        self.waiting: List[Request] = []
+        self.running: List[Request] = []
+        self._next_id = 1
+        self._prefer_decode = False
+        self.perf = get_perf_stats()
+        self._graphs: Dict[int, Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        if self.hybrid:
+            # per-layer cache geometry comes from the model's mixers; every
+            # live sequence also owns one slot of recurrent/convolution state
+            self.kv = PagedKVCache(
+                self.spec.num_layers, 0, 0, self.block_size, num_blocks, self.device,
+                self.dtype, layer_shapes=self.model.kv_layer_shapes(),
+                prefix_caching=False,
+            )
+            self.state_pool = StateSlotPool(
+                int(cfg.get("state_slots", self.max_batch)),
+                self.model.state_layer_shapes(), self.device,
+            )
+            self.max_blocks_per_seq = (
+                min(self.max_seq_len, num_blocks * self.block_size) + self.block_size - 1
+            ) // self.block_size
+            self._dec_ws = None
+            return
         hk_local = self.spec.num_kv_heads // self.tp
         self.kv = PagedKVCache(
             self.spec.num_layers, hk_local, self.spec.head_dim,
@@ -299,24 +350,23 @@ class LLMEngine:
             )
         else:
             self._dec_ws = None
-        self._graphs: Dict[int, Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
-
-        self.requests: Dict[int, Request] = {}
-        self.waiting: List[Request] = []
-        self.running: List[Request] = []
-        self._next_id = 1
-        self._prefer_decode = False
-        self.perf = get_perf_stats()
 
     # ------------------------------------------------------------------
     def _pick_num_blocks(self, cfg: dict) -> int:
         if cfg.get("kv_num_blocks"):
             return int(cfg["kv_num_blocks"])
         kv_gb = float(cfg.get("kv_cache_gb", 0) or 0)
-        hk_local = self.spec.num_kv_heads // self.tp
-        block_bytes = (
-            2 * self.spec.num_layers * self.block_size * hk_local * self.spec.head_dim * 2
-        )
+        if self.hybrid:
+            esz = 4 if self.dtype == torch.float32 else 2
+            per_token = sum(
+                sh[0] * (sh[1] + sh[2]) for sh in self.model.kv_layer_shapes() if sh
+            )
+            block_bytes = max(1, per_token * self.block_size * esz)
+        else:
+            hk_local = self.spec.num_kv_heads // self.tp
+            block_bytes = (
+                2 * self.spec.num_layers * self.block_size * hk_local * self.spec.head_dim * 2
+            )
         if self.device == "cpu":
             blocks_needed = self.max_batch * (
                 (self.max_seq_len + self.block_size - 1) // self.block_size
@@ -488,12 +538,18 @@ class LLMEngine:
             needed = (len(req.prompt_ids) + self.block_size - 1) // self.block_size + 1
             if self.running and self.kv.num_free() < needed:
                 break
+            if self.state_pool is not None and self.state_pool.num_free() == 0:
+                break  # every state slot is held by a live sequence
             self.waiting.pop(0)
-            req.seq = SequenceState(self.kv, req.prompt_ids)
+            req.seq = SequenceState(self.kv, req.prompt_ids, self.state_pool)
             reused = req.seq.reuse_prefix()
             req.prefill_done = reused
             self.perf.record_metric("engine_prefix_reused_tokens", float(reused))
             self.running.append(req)
+
+        if self.hybrid:
+            self._step_mixed()
+            return
 
         # speculative proposals awaiting their verify forward
         spec = next(
@@ -564,6 +620,162 @@ class LLMEngine:
         req.prefill_done = 0
         self.waiting.insert(0, req)
         self.perf.record_metric("engine_preemptions", 1.0)
+
+    # -- flat multi-sequence steps (hybrid models) -------------------------
+    @torch.inference_mode()
+    def _forward_mixed(self, work: List[Tuple[Request, int, int]]) -> torch.Tensor:
+        """ONE forward over prompt portions and decoded tokens of several
+        sequences: work = [(request, start, count)] feeds tokens
+        [start, start+count) of each request's sequence, continuing from the
+        paged keys/values and the state slot that earlier steps left.
+        Capacity for start+count tokens must already be ensured. Returns the
+        model's hidden rows [sum(count), C] in work order and marks the
+        tokens cached."""
+        from opsagent_amd.ops.mixer_ops import SeqBatch
+
+        ids: List[int] = []
+        chunks = []
+        for req, start, count in work:
+            seq = req.seq
+            assert start == seq.num_cached and start + count <= len(seq.token_ids)
+            ids.extend(seq.token_ids[start : start + count])
+            chunks.append((start, count, seq.state_slot, seq.blocks))
+        pure_decode = all(c[1] == 1 for c in chunks)
+        if (
+            pure_decode and self.device == "cuda" and self.use_hipgraph
+            and len(chunks) <= self.max_batch
+        ):
+            hidden = self._mixed_decode_graphed(ids, chunks)
+        else:
+            sb = SeqBatch.build(chunks, self.block_size, self.device)
+            fb = ForwardBatch(
+                kind="mixed",
+                input_ids=torch.tensor(ids, dtype=torch.int64).to(self.device),
+                positions=None,
+                slot_mapping=sb.slot_mapping,
+                seq_batch=sb,
+            )
+            hidden = self.model(fb, self.kv.layers, self.state_pool.tensors)
+        for req, start, count in work:
+            req.seq.num_cached = start + count
+        return hidden
+
+    def _mixed_decode_graphed(self, ids: List[int], chunks) -> torch.Tensor:
+        """Decode-only step of a hybrid model through a hipGraph captured per
+        batch bucket: static SeqBatch tensors are refilled, padding rows
+        repeat row 0 (same token, same slots: an idempotent rewrite is NOT
+        safe for recurrent state, so padded rows get count 0 instead)."""
+        from opsagent_amd.ops.mixer_ops import SeqBatch
+
+        B = len(chunks)
+        bucket = self._bucket(B)
+        ent = self._graphs.get(bucket)
+        if ent is None:
+            dev = self.device
+            i32 = torch.int32
+            sb = SeqBatch(
+                cu=list(range(bucket + 1)), past=[0] * bucket, slots=[0] * bucket,
+                cu_t=torch.zeros(bucket + 1, dtype=i32, device=dev),
+                past_t=torch.zeros(bucket, dtype=i32, device=dev),
+                slots_t=torch.zeros(bucket, dtype=i32, device=dev),
+                seq_of_t=torch.arange(bucket, dtype=i32, device=dev),
+                slot_mapping=torch.zeros(bucket, dtype=i32, device=dev),
+                block_table=torch.zeros(bucket, self.max_blocks_per_seq, dtype=i32, device=dev),
+                max_chunk=1,
+                max_total=self.max_blocks_per_seq * self.block_size,
+            )
+            ids_t = torch.zeros(bucket, dtype=torch.int64, device=dev)
+            ent = {"sb": sb, "ids": ids_t, "graph": None, "out": None}
+            self._graphs[bucket] = ent
+        sb, ids_t = ent["sb"], ent["ids"]
+        # host staging -> static device tensors. Padding rows: zero tokens
+        # (cu stays flat), so no kernel touches any state for them.
+        cu = [min(i, B) for i in range(bucket + 1)]
+        past = [c[0] for c in chunks] + [0] * (bucket - B)
+        slots = [c[2] for c in chunks] + [0] * (bucket - B)
+        bs = self.block_size
+        slot_map = [c[3][c[0] // bs] * bs + c[0] % bs for c in chunks]
+        slot_map += [slot_map[0]] * (bucket - B)
+        seq_of = list(range(B)) + [0] * (bucket - B)
+        bt = torch.zeros(bucket, self.max_blocks_per_seq, dtype=torch.int32)
+        for b, c in enumerate(chunks):
+            bt[b, : len(c[3])] = torch.tensor(c[3], dtype=torch.int32)
+        # sb's HOST lists stay at the bucket's upper bound (one token per
+        # row): they only size launches; the kernels read the device copies
+        sb.cu_t.copy_(torch.tensor(cu, dtype=torch.int32))
+        sb.past_t.copy_(torch.tensor(past, dtype=torch.int32))
+        sb.slots_t.copy_(torch.tensor(slots, dtype=torch.int32))
+        sb.seq_of_t.copy_(torch.tensor(seq_of, dtype=torch.int32))
+        sb.slot_mapping.copy_(torch.tensor(slot_map, dtype=torch.int32))
+        sb.block_table.copy_(bt)
+        ids_t.copy_(torch.tensor(ids + [ids[0]] * (bucket - B), dtype=torch.int64))
+        fb = ForwardBatch(kind="mixed", input_ids=ids_t, positions=None,
+                          slot_mapping=sb.slot_mapping, seq_batch=sb)
+        if ent["graph"] is None:
+            # first use of the bucket runs eagerly once (library warm-up,
+            # allocator) and captures from the SECOND use on: the eager run
+            # has already advanced the recurrent state for this step
+            if ent["out"] is None:
+                ent["out"] = "warm"
+                return self.model(fb, self.kv.layers, self.state_pool.tensors)[:B]
+            try:
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    out = self.model(fb, self.kv.layers, self.state_pool.tensors)
+                # capture does not execute: replay performs this step
+                ent["graph"], ent["out"] = g, out
+                log.info("captured hybrid decode hipGraph for batch bucket %d", bucket)
+            except Exception:  # noqa: BLE001 — capture failure must not kill serving
+                log.exception("hipGraph capture failed for hybrid bucket %d — eager decode", bucket)
+                self.use_hipgraph = False
+                torch.cuda.synchronize()
+                return self.model(fb, self.kv.layers, self.state_pool.tensors)[:B]
+        ent["graph"].replay()
+        return ent["out"][:B]
+
+    def _step_mixed(self) -> None:
+        """Scheduler step of a hybrid model: every running request advances
+        in the SAME forward — requests still reading their prompt (or owing
+        fast-forwarded tokens) contribute a portion under a shared token
+        budget, decoding requests one token each."""
+        t0 = time.perf_counter()
+        work: List[Tuple[Request, int, int]] = []
+        budget = self.max_prefill_chunk
+        for req in list(self.running):
+            if req.finished:
+                continue
+            seq = req.seq
+            pending = len(seq.token_ids) - seq.num_cached
+            count = 1 if pending == 1 else min(pending, budget)
+            if count <= 0:
+                continue
+            try:
+                seq.ensure_capacity(seq.num_cached + count)
+            except BlockAllocatorError:
+                self._preempt(req)
+                continue
+            if pending > 1:
+                budget -= count
+            work.append((req, seq.num_cached, count))
+        if not work:
+            self._reap()
+            return
+        hidden = self._forward_mixed(work)
+        rows, batch, off = [], [], 0
+        for req, start, count in work:
+            off += count
+            req.prefill_done = min(len(req.prompt_ids), req.seq.num_cached)
+            if req.seq.num_cached == len(req.seq.token_ids):
+                rows.append(off - 1)
+                batch.append(req)
+        if batch:
+            idx = torch.tensor(rows, dtype=torch.int64).to(self.device)
+            logits = self.model.compute_logits(hidden.index_select(0, idx))
+            self._sample_and_append(batch, logits)
+        self._reap()
+        self.perf.record_metric("engine_mixed_step_ms", (time.perf_counter() - t0) * 1000.0)
+        self.perf.record_metric("engine_mixed_step_tokens", float(off))
 
     # -- prefill ---------------------------------------------------------
     @torch.inference_mode()
@@ -1161,7 +1373,11 @@ class LLMEngine:
         needs = any(r.params.needs_logit_transform() for r in batch)
         if self.device == "cuda":
             lg = logits.contiguous()
-            if needs:
+            if lg.dtype == torch.float32:
+                # float32 logits (hybrid models) are sampled in float32
+                if needs:
+                    lg = self._transform_logits(batch, lg.clone()).contiguous()
+            elif needs:
                 lg = (
                     self._transform_logits(batch, lg.float())
                     .to(torch.bfloat16)

@@ -36,17 +36,30 @@ class PagedKVCache:
         num_blocks: int,
         device: str,
         dtype: torch.dtype = torch.bfloat16,
+        layer_shapes: Optional[Sequence[Optional[Tuple[int, int, int]]]] = None,
+        prefix_caching: bool = True,
     ):
+        """layer_shapes (optional) gives each layer's own (kv_heads, key dim,
+        value dim), or None for a layer that keeps no keys and values (a
+        recurrent mixer); without it every layer is [kv_heads, head_dim] for
+        both. prefix_caching=False turns block publishing and reuse off: a
+        model that also carries recurrent state cannot restart from cached
+        keys alone."""
         assert block_size & (block_size - 1) == 0, "block_size must be a power of 2"
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.device = device
-        self.layers: List[Tuple[torch.Tensor, torch.Tensor]] = []
-        for _ in range(num_layers):
-            k = torch.zeros(
-                num_blocks, block_size, num_kv_heads_local, head_dim, dtype=dtype, device=device
-            )
-            v = torch.zeros_like(k)
+        self.prefix_caching = prefix_caching
+        self.layers: List[Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]] = []
+        if layer_shapes is None:
+            layer_shapes = [(num_kv_heads_local, head_dim, head_dim)] * num_layers
+        for shape in layer_shapes:
+            if shape is None:
+                self.layers.append((None, None))
+                continue
+            hk, kdim, vdim = shape
+            k = torch.zeros(num_blocks, block_size, hk, kdim, dtype=dtype, device=device)
+            v = torch.zeros(num_blocks, block_size, hk, vdim, dtype=dtype, device=device)
             self.layers.append((k, v))
         # allocator state
         self._free: collections.deque[int] = collections.deque(range(num_blocks))
@@ -115,6 +128,8 @@ class PagedKVCache:
         bs = self.block_size
         blocks: List[int] = []
         h = 0
+        if not self.prefix_caching:
+            return blocks, 0
         max_full = (len(token_ids) - 1) // bs  # leave ≥1 token to prefill
         for i in range(max_full):
             h = self.chain_hash(h, token_ids[i * bs : (i + 1) * bs])
@@ -151,11 +166,55 @@ class PagedKVCache:
         return bid
 
 
+class StateSlotPool:
+    """Fixed-size per-sequence state beside the paged keys and values: the
+    recurrent matrix of a delta-rule mixer and the last inputs of causal
+    short convolutions. One slot per live sequence; a slot is handed out at
+    admission and returned when the sequence ends or is preempted.
+
+    A slot is NOT cleared when it is reused: every kernel that reads state
+    takes the sequence's start position and treats everything before
+    position 0 as zero, so stale contents are never observed (and nothing
+    has to be memset inside a captured graph).
+
+    tensors[layer][name] is [num_slots, *shape] float32.
+    """
+
+    def __init__(self, num_slots: int, layer_shapes: Sequence[Dict[str, Tuple[int, ...]]],
+                 device: str):
+        self.num_slots = num_slots
+        self.tensors: List[Dict[str, torch.Tensor]] = []
+        for shapes in layer_shapes:
+            self.tensors.append({
+                name: torch.zeros(num_slots, *shape, dtype=torch.float32, device=device)
+                for name, shape in shapes.items()
+            })
+        self._free: collections.deque[int] = collections.deque(range(num_slots))
+
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def alloc(self) -> int:
+        if not self._free:
+            raise BlockAllocatorError("out of state slots")
+        return self._free.popleft()
+
+    def release(self, slot: int) -> None:
+        assert 0 <= slot < self.num_slots and slot not in self._free
+        self._free.append(slot)
+
+
 class SequenceState:
     """Per-sequence cache bookkeeping."""
 
-    def __init__(self, cache: PagedKVCache, token_ids: List[int]):
+    def __init__(self, cache: PagedKVCache, token_ids: List[int],
+                 state_pool: Optional[StateSlotPool] = None):
         self.cache = cache
+        self.state_pool = state_pool
+        # recurrent/convolution state slot (None for pure-attention models)
+        self.state_slot: Optional[int] = (
+            state_pool.alloc() if state_pool is not None else None
+        )
         self.token_ids = list(token_ids)  # prompt + generated
         self.blocks: List[int] = []
         self.num_cached = 0     # tokens whose KV is in cache
@@ -194,6 +253,8 @@ class SequenceState:
 
     def publish_full_blocks(self) -> None:
         """Publish newly-completed full blocks to the prefix cache."""
+        if not self.cache.prefix_caching:
+            return
         bs = self.cache.block_size
         full = self.num_cached // bs
         while self.published < full:
@@ -211,3 +272,6 @@ class SequenceState:
         for bid in self.blocks:
             self.cache.release(bid)
         self.blocks = []
+        if self.state_slot is not None:
+            self.state_pool.release(self.state_slot)
+            self.state_slot = None

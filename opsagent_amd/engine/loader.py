@@ -128,6 +128,11 @@ def load_weights(model: LlamaForCausalLM, path: str) -> int:
     sharded HF index, or directory) into the model, slicing TP shards.
     Returns the number of parameters loaded."""
     raw = _load_checkpoint(path)
+    if hasattr(model, "load_named_tensors"):
+        # architectures with their own tensor names fill themselves
+        n = model.load_named_tensors(raw)
+        log.info("loaded %d tensors from %s", n, path)
+        return n
     tensors = {_canonical_from_hf(k): v for k, v in raw.items()}
     spec = model.spec
     tp, rank = get_tp_size(), get_tp_rank()

@@ -68,6 +68,9 @@ class ForwardBatch:
     seq_lens: Optional[torch.Tensor] = None     # [B] int32
     decode_workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
     nsplit: Optional[int] = None
+    # kind == "mixed": a flat multi-sequence step (prompt portions beside
+    # decoded tokens); geometry in an ops.mixer_ops.SeqBatch
+    seq_batch: Optional[object] = None
 
 
 def _shard(t: torch.Tensor, dim: int, rank: int, size: int) -> torch.Tensor:

@@ -27,6 +27,16 @@ SOURCES = [
     "moe_gemv.hip",
 ]
 
+# the sequence-mixer kernels of hybrid decoders live in a library of their
+# own: a checkout that serves only such a model compiles just what it loads
+MIXER_SOURCES = ["mixers.hip"]
+MIXER_OUT = os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "libopsagent_mixers.so"
+)
+
+# packed-fp32 VALU forms are switched off for every kernel
+HIP_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
 HIPCC = os.environ.get("HIPCC", "hipcc")
 ARCH = os.environ.get("OPSAGENT_GPU_ARCH", "gfx950")
 
@@ -43,37 +53,64 @@ def _mtime(path: str) -> float:
         return 0.0
 
 
-def needs_rebuild() -> bool:
-    out_t = _mtime(OUT)
+def needs_rebuild(out: str = OUT, sources=None) -> bool:
+    out_t = _mtime(out)
     if out_t == 0.0:
         return True
-    deps = [os.path.join(CSRC, s) for s in SOURCES] + [os.path.join(CSRC, "common.h")]
+    deps = [os.path.join(CSRC, s) for s in (sources or SOURCES)]
+    deps.append(os.path.join(CSRC, "common.h"))
     return any(_mtime(d) > out_t for d in deps)
+
+
+def _compile_library(sources, out: str, verbose: bool) -> str:
+    """Compile each source to an object (in parallel), then link. The
+    library is written under a temporary name and renamed into place, so a
+    concurrent process never loads a half-written file."""
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+
+    tmp = tempfile.mkdtemp(prefix="opsagent_build_")
+    base = [HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", *HIP_FLAGS]
+
+    def one(src: str) -> str:
+        obj = os.path.join(tmp, src + ".o")
+        cmd = base + ["-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print("[opsagent build]", " ".join(cmd), file=sys.stderr)
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(
+                f"hipcc failed ({proc.returncode}) on {src}:\n{proc.stdout}\n{proc.stderr}"
+            )
+        return obj
+
+    try:
+        jobs = max(1, min(len(sources), int(os.environ.get("MAX_JOBS", "8"))))
+        with ThreadPoolExecutor(jobs) as pool:
+            objs = list(pool.map(one, sources))
+        part = out + f".{os.getpid()}.part"
+        cmd = [HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", part, *objs]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"link failed ({proc.returncode}):\n{proc.stdout}\n{proc.stderr}")
+        os.replace(part, out)
+    finally:
+        import shutil
+
+        shutil.rmtree(tmp, ignore_errors=True)
+    return out
 
 
 def build(verbose: bool = True, force: bool = False) -> str:
     if not force and not needs_rebuild():
         return OUT
-    srcs = [os.path.join(CSRC, s) for s in SOURCES]
-    cmd = [
-        HIPCC,
-        f"--offload-arch={ARCH}",
-        "-O3",
-        "-std=c++17",
-        "-shared",
-        "-fPIC",
-        "-o",
-        OUT,
-        *srcs,
-    ]
-    if verbose:
-        print("[opsagent build]", " ".join(cmd), file=sys.stderr)
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(
-            f"hipcc failed ({proc.returncode}):\n{proc.stdout}\n{proc.stderr}"
-        )
-    return OUT
+    return _compile_library(SOURCES, OUT, verbose)
+
+
+def build_mixers(verbose: bool = True, force: bool = False) -> str:
+    if not force and not needs_rebuild(MIXER_OUT, MIXER_SOURCES):
+        return MIXER_OUT
+    return _compile_library(MIXER_SOURCES, MIXER_OUT, verbose)
 
 
 def build_grammar(verbose: bool = True, force: bool = False) -> str:
@@ -92,9 +129,11 @@ def build_grammar(verbose: bool = True, force: bool = False) -> str:
 def build_all(force: bool = False) -> None:
     build_grammar(force=force)
     build(force=force)
+    build_mixers(force=force)
 
 
 if __name__ == "__main__":
     build_all(force="--force" in sys.argv)
     print(OUT)
+    print(MIXER_OUT)
     print(GRAMMAR_OUT)

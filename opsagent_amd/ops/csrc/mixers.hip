@@ -1,0 +1,801 @@
+// Sequence-mixer kernels for hybrid decoders on MI355X (gfx950): grouped RMS
+// norm onto a float32 residual, causal short convolutions with carried
+// inputs, softmax attention with a per-head linear distance penalty over
+// the paged cache (separate key and value sizes, per-head output gate), and
+// the gated delta rule with one decay per head and key channel.
+//
+// Every kernel works on a FLAT multi-sequence batch: T new tokens of B
+// sequences laid end to end. cu[b]..cu[b+1] are sequence b's tokens, which
+// continue it from position past[b]; slots[b] is its row in the state
+// tensors; seq_of[t] is the sequence of token t. A prompt portion and a
+// single decoded token are the same case with different counts.
+//
+// Precision: norms, softmax scores and weights, decays, gates, the
+// recurrent state and the residual are float32 whatever the activation
+// type is. Activations/weights are bf16 (dt = 0) or float32 (dt = 1).
+//
+// All sizes are run-time values; nothing assumes a multiple of 64.
+
+#include "common.h"
+
+#include <algorithm>
+
+typedef uint16_t bf16s;  // bf16 storage
+
+__device__ __forceinline__ float ldf(const float* p, int64_t i) { return p[i]; }
+__device__ __forceinline__ float ldf(const bf16s* p, int64_t i) { return bf16_to_f32(p[i]); }
+__device__ __forceinline__ void stf(float* p, int64_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void stf(bf16s* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplusf_(float z) {
+    return fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z)));
+}
+
+// ---------------------------------------------------------------------------
+// Causal convolution over time, per channel, continued from carried inputs.
+//   y_t = sum_j w[c, j] * x_(t - taps + 1 + j)   (+ x_t) (-> silu)
+// Inputs at positions < 0 are zero. state[slot, i, c] (float32) holds the
+// input at position past - (taps-1) + i.
+template <typename TI, typename TW, typename TO>
+__global__ __launch_bounds__(256) void causal_conv_kernel(
+    const TI* __restrict__ x, int64_t xs, const TW* __restrict__ w,
+    const float* __restrict__ state, TO* __restrict__ out, int64_t os,
+    const int* __restrict__ seq_of, const int* __restrict__ cu,
+    const int* __restrict__ past, const int* __restrict__ slots, int T, int C,
+    int taps, int add_input, int act_silu) {
+    const int64_t total = (int64_t)T * C;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int t = (int)(idx / C), c = (int)(idx % C);
+        const int b = seq_of[t];
+        const int lo = cu[b];
+        const int local = t - lo;
+        const int pos = past[b] + local;
+        const float* st = state + (int64_t)slots[b] * (taps - 1) * C;
+        float acc = 0.0f;
+        for (int j = 0; j < taps; ++j) {
+            const int d = j - (taps - 1);  // <= 0
+            if (pos + d < 0) continue;
+            const int s = local + d;
+            float xv = (s >= 0) ? ldf(x, (int64_t)(lo + s) * xs + c)
+                                : st[(int64_t)(taps - 1 + s) * C + c];
+            acc += ldf(w, (int64_t)c * taps + j) * xv;
+        }
+        if (add_input) acc += ldf(x, (int64_t)t * xs + c);
+        if (act_silu) acc = acc * sigmoidf_(acc);
+        stf(out, (int64_t)t * os + c, acc);
+    }
+}
+
+// After the convolution: carry the last taps-1 inputs of every sequence.
+// One thread per (sequence, channel) walks the entries in ascending order,
+// so a shifted old entry is read before it is overwritten.
+template <typename TI>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    const TI* __restrict__ x, int64_t xs, float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ past,
+    const int* __restrict__ slots, int B, int C, int taps) {
+    const int64_t total = (int64_t)B * C;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int b = (int)(idx / C), c = (int)(idx % C);
+        const int lo = cu[b], n = cu[b + 1] - lo;
+        if (n <= 0) continue;
+        const int p = past[b];
+        float* st = state + (int64_t)slots[b] * (taps - 1) * C;
+        for (int i = 0; i < taps - 1; ++i) {
+            const int local = n - (taps - 1) + i;
+            float v;
+            if (local >= 0) v = ldf(x, (int64_t)(lo + local) * xs + c);
+            else v = (p + local < 0) ? 0.0f : st[(int64_t)(i + n) * C + c];
+            st[(int64_t)i * C + c] = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// RMS norm in `groups` consecutive parts, times w; one block per token, one
+// wave per part. residual (float32, may be null) is updated in place:
+// residual += norm(y) * w; `copy` (may be null) gets the result in the
+// activation type.
+template <typename TY, typename TW, typename TO>
+__global__ __launch_bounds__(256) void group_rmsnorm_kernel(
+    const TY* __restrict__ y, int64_t ys, const TW* __restrict__ w,
+    float* __restrict__ residual, TO* __restrict__ copy, int C, int groups,
+    float eps) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int gs = C / groups;
+    for (int g = wave; g < groups; g += nw) {
+        const int64_t base = (int64_t)t * ys + (int64_t)g * gs;
+        float ss = 0.0f;
+        for (int i = lane; i < gs; i += 64) {
+            float v = ldf(y, base + i);
+            ss += v * v;
+        }
+        ss = wave_reduce_sum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)gs + eps);
+        for (int i = lane; i < gs; i += 64) {
+            const int c = g * gs + i;
+            float v = ldf(y, base + i) * r * ldf(w, c);
+            if (residual) {
+                v += residual[(int64_t)t * C + c];
+                residual[(int64_t)t * C + c] = v;
+            }
+            if (copy) stf(copy, (int64_t)t * C + c, v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Attention input preparation, one block per token: the projection biases
+// are added (bias over q | k | v columns, may be null), then weighted RMS
+// norm over the WHOLE q projection and over the whole k projection and an
+// unweighted RMS norm of each value head; q goes to q_out, k and v to their
+// cache slot.
+template <typename TC>
+__global__ __launch_bounds__(256) void attn_prepare_kernel(
+    const TC* __restrict__ qkv, int64_t qs, const TC* __restrict__ bias,
+    const TC* __restrict__ qw, const TC* __restrict__ kw, TC* __restrict__ q_out,
+    TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+    const int* __restrict__ slot_mapping, const int* __restrict__ cu, int B, int H,
+    int G, int D, int Dv, float eps) {
+    __shared__ float red[8];
+    const int t = blockIdx.x;
+    if (t >= cu[B]) return;  // padding row of a fixed-size (captured) launch
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const TC* row = qkv + (int64_t)t * qs;
+    const int nq = H * D, nk = G * D;
+    const int64_t slot = slot_mapping[t];
+    auto val = [&](int i) { return ldf(row, i) + (bias ? ldf(bias, i) : 0.0f); };
+    float sq = 0.0f, sk = 0.0f;
+    for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+        float v = val(i);
+        sq += v * v;
+    }
+    for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+        float v = val(nq + i);
+        sk += v * v;
+    }
+    sq = wave_reduce_sum(sq);
+    sk = wave_reduce_sum(sk);
+    if (lane == 0) {
+        red[wave] = sq;
+        red[4 + wave] = sk;
+    }
+    __syncthreads();
+    sq = 0.0f;
+    sk = 0.0f;
+    for (int i = 0; i < nw; ++i) {
+        sq += red[i];
+        sk += red[4 + i];
+    }
+    const float rq = 1.0f / sqrtf(sq / (float)nq + eps);
+    const float rk = 1.0f / sqrtf(sk / (float)nk + eps);
+    for (int i = threadIdx.x; i < nq; i += blockDim.x)
+        stf(q_out, (int64_t)t * nq + i, val(i) * rq * ldf(qw, i));
+    for (int i = threadIdx.x; i < nk; i += blockDim.x)
+        stf(k_cache, slot * nk + i, val(nq + i) * rk * ldf(kw, i));
+    for (int g = wave; g < G; g += nw) {
+        const int off = nq + nk + g * Dv;
+        float sv = 0.0f;
+        for (int i = lane; i < Dv; i += 64) {
+            float v = val(off + i);
+            sv += v * v;
+        }
+        sv = wave_reduce_sum(sv);
+        const float rv = 1.0f / sqrtf(sv / (float)Dv + eps);
+        for (int i = lane; i < Dv; i += 64)
+            stf(v_cache, slot * (int64_t)(G * Dv) + g * Dv + i, val(off + i) * rv);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Softmax attention with a linear distance penalty over the paged cache.
+//   score(i, j) = q_i . k_j * scale - slope_h * (i - j),  j <= i
+//   out_i,h = sigmoid(gate_i,h) * sum_j softmax_j(score) v_j
+// grid = (query tiles, kv heads, key splits). A tile is up to TQ
+// consecutive new tokens of ONE sequence with all R = H/G query heads of
+// the kv head: ROWS = TQ*R rows share every staged key/value tile. Each of
+// the 4 waves owns rows wave, wave+4, ...; in the score phase a lane is a
+// key, in the value phase a lane is a value channel. Keys KT at a time go
+// through LDS (K padded to an odd word stride).
+// With nsplit > 1 a block covers every nsplit-th key tile and writes
+// unnormalised partials (acc, m, l) that attn_combine_kernel merges.
+#define ATT_MAXR 4   // rows per wave
+#define ATT_MAXV 4   // value channels per lane (Dv <= 256)
+
+template <typename TC>
+__global__ __launch_bounds__(256) void attn_bias_paged_kernel(
+    const TC* __restrict__ q, const TC* __restrict__ gate, int64_t gs,
+    const TC* __restrict__ k_cache, const TC* __restrict__ v_cache,
+    TC* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int* __restrict__ cu, const int* __restrict__ past,
+    const int* __restrict__ block_table, int max_blocks, int block_size,
+    const float* __restrict__ slopes, int B, int H, int G, int D, int Dv, int TQ,
+    int KT, int kstride, float scale, int nsplit) {
+    extern __shared__ float lds[];
+    const int R = H / G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = blockIdx.y, split = blockIdx.z;
+    // locate this block's tile: walk the sequences
+    int tile = blockIdx.x, b = 0, lo = 0, n = 0;
+    for (; b < B; ++b) {
+        lo = cu[b];
+        n = cu[b + 1] - lo;
+        const int nt = (n + TQ - 1) / TQ;
+        if (tile < nt) break;
+        tile -= nt;
+    }
+    if (b >= B) return;
+    const int t0 = tile * TQ;                       // local offset in the portion
+    const int nq_tok = min(TQ, n - t0);
+    const int rows = nq_tok * R;
+    const int p0 = past[b] + t0;                    // position of the first query
+    const int last_pos = p0 + nq_tok - 1;
+    const int* bt = block_table + (int64_t)b * max_blocks;
+
+    float* Qs = lds;                                // [TQ*R][D]
+    float* Ps = Qs + (size_t)TQ * R * D;            // [4][KT]
+    TC* Ks = (TC*)(Ps + 4 * KT);                    // [KT][kstride]
+    TC* Vs = Ks + (size_t)KT * kstride;             // [KT][Dv]
+
+    for (int i = threadIdx.x; i < rows * D; i += blockDim.x) {
+        const int r = i / D, d = i % D;
+        const int tok = lo + t0 + r / R, h = g * R + r % R;
+        Qs[i] = ldf(q, ((int64_t)tok * H + h) * D + d) * scale;
+    }
+    float m[ATT_MAXR], l[ATT_MAXR], acc[ATT_MAXR][ATT_MAXV];
+#pragma unroll
+    for (int i = 0; i < ATT_MAXR; ++i) {
+        m[i] = -INFINITY;
+        l[i] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < ATT_MAXV; ++c) acc[i][c] = 0.0f;
+    }
+    const int nkt = last_pos / KT + 1;
+    for (int kt = split; kt < nkt; kt += nsplit) {
+        const int k0 = kt * KT;
+        const int nk = min(KT, last_pos + 1 - k0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < nk * D; i += blockDim.x) {
+            const int j = i / D, d = i % D;
+            const int key = k0 + j;
+            const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
+            Ks[j * kstride + d] = k_cache[(slot * G + g) * D + d];
+        }
+        for (int i = threadIdx.x; i < nk * Dv; i += blockDim.x) {
+            const int j = i / Dv, d = i % Dv;
+            const int key = k0 + j;
+            const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
+            Vs[j * Dv + d] = v_cache[(slot * G + g) * Dv + d];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ri = 0; ri < ATT_MAXR; ++ri) {
+            const int r = wave + 4 * ri;
+            if (r >= rows) break;
+            const int pos = p0 + r / R;
+            if (k0 > pos) continue;
+            const float slope = slopes[g * R + r % R];
+            float s = -INFINITY;
+            if (lane < nk && k0 + lane <= pos) {
+                const float* qr = Qs + r * D;
+                const TC* kr = Ks + lane * kstride;
+                float a = 0.0f;
+                for (int d = 0; d < D; ++d) a += qr[d] * ldf(kr, d);
+                s = a - slope * (float)(pos - (k0 + lane));
+            }
+            const float mx = fmaxf(m[ri], wave_reduce_max(s));
+            const float p = (s == -INFINITY) ? 0.0f : expf(s - mx);
+            const float corr = (m[ri] == -INFINITY) ? 0.0f : expf(m[ri] - mx);
+            l[ri] = l[ri] * corr + wave_reduce_sum(p);
+            m[ri] = mx;
+            if (lane < KT) Ps[wave * KT + lane] = p;
+            // a wave's lanes run in lockstep; LDS writes of this wave are
+            // visible to it after the wait below
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            __builtin_amdgcn_wave_barrier();
+            const int jmax = min(nk, pos - k0 + 1);
+#pragma unroll
+            for (int c = 0; c < ATT_MAXV; ++c) {
+                const int ch = lane + 64 * c;
+                float a = acc[ri][c] * corr;
+                if (ch < Dv)
+                    for (int j = 0; j < jmax; ++j) a += Ps[wave * KT + j] * ldf(Vs, j * Dv + ch);
+                acc[ri][c] = a;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+#pragma unroll
+    for (int ri = 0; ri < ATT_MAXR; ++ri) {
+        const int r = wave + 4 * ri;
+        if (r >= rows) break;
+        const int tok = lo + t0 + r / R, h = g * R + r % R;
+        if (nsplit == 1) {
+            const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h));
+            const float inv = gt / l[ri];
+#pragma unroll
+            for (int c = 0; c < ATT_MAXV; ++c) {
+                const int ch = lane + 64 * c;
+                if (ch < Dv) stf(out, ((int64_t)tok * H + h) * Dv + ch, acc[ri][c] * inv);
+            }
+        } else {
+            const int64_t pr = ((int64_t)tok * H + h) * nsplit + split;
+#pragma unroll
+            for (int c = 0; c < ATT_MAXV; ++c) {
+                const int ch = lane + 64 * c;
+                if (ch < Dv) part_o[pr * Dv + ch] = acc[ri][c];
+            }
+            if (lane == 0) {
+                part_ml[pr * 2] = m[ri];
+                part_ml[pr * 2 + 1] = l[ri];
+            }
+        }
+    }
+}
+
+// merge key-split partials: one wave per (token, head)
+template <typename TC>
+__global__ __launch_bounds__(64) void attn_combine_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    const TC* __restrict__ gate, int64_t gs, TC* __restrict__ out, int H, int Dv,
+    int nsplit) {
+    const int64_t row = blockIdx.x;  // tok * H + h
+    const int tok = (int)(row / H), h = (int)(row % H);
+    const int lane = threadIdx.x;
+    float mx = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part_ml[(row * nsplit + s) * 2]);
+    float l = 0.0f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float ms = part_ml[(row * nsplit + s) * 2];
+        if (ms != -INFINITY) l += part_ml[(row * nsplit + s) * 2 + 1] * expf(ms - mx);
+    }
+    const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) / l;
+    for (int ch = lane; ch < Dv; ch += 64) {
+        float a = 0.0f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float ms = part_ml[(row * nsplit + s) * 2];
+            if (ms != -INFINITY) a += part_o[(row * nsplit + s) * Dv + ch] * expf(ms - mx);
+        }
+        stf(out, row * Dv + ch, a * gt);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Delta-rule preparation, one block per token (all float32 outputs):
+//   qn = q / sqrt(sum q^2 + 1e-6) * D^-1/2,  kn = k / sqrt(sum k^2 + 1e-6)
+//   decay[h, d] = exp(-exp(A_log[h]) * softplus(a[h, d] + dt_bias[h, d]))
+//   beta[h] = sigmoid(b[h])
+template <typename TC>
+__global__ __launch_bounds__(256) void delta_prepare_kernel(
+    const TC* __restrict__ q, int64_t qs, const TC* __restrict__ k, int64_t ks,
+    const TC* __restrict__ bl, int64_t bs, const TC* __restrict__ a, int64_t as,
+    const TC* __restrict__ dt_bias, const TC* __restrict__ a_log,
+    float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ decay,
+    float* __restrict__ beta, int H, int G, int D) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const float qscale = 1.0f / sqrtf((float)D);
+    for (int u = wave; u < 2 * G; u += nw) {
+        const int g = u >> 1;
+        const bool is_q = (u & 1) == 0;
+        const TC* src = is_q ? q + (int64_t)t * qs + g * D : k + (int64_t)t * ks + g * D;
+        float* dst = (is_q ? qn : kn) + ((int64_t)t * G + g) * D;
+        float ss = 0.0f;
+        for (int i = lane; i < D; i += 64) {
+            float v = ldf(src, i);
+            ss += v * v;
+        }
+        ss = wave_reduce_sum(ss);
+        const float r = (1.0f / sqrtf(ss + 1e-6f)) * (is_q ? qscale : 1.0f);
+        for (int i = lane; i < D; i += 64) dst[i] = ldf(src, i) * r;
+    }
+    for (int i = threadIdx.x; i < H * D; i += blockDim.x) {
+        const int h = i / D;
+        const float z = ldf(a, (int64_t)t * as + i) + ldf(dt_bias, i);
+        decay[(int64_t)t * H * D + i] = expf(-expf(ldf(a_log, h)) * softplusf_(z));
+    }
+    for (int h = threadIdx.x; h < H; h += blockDim.x)
+        beta[(int64_t)t * H + h] = sigmoidf_(ldf(bl, (int64_t)t * bs + h));
+}
+
+// The recurrence. grid = (sequences, heads, value-column groups of 16), one
+// wave per block. Lane = (column, row group): 16 columns x 4 row groups,
+// each lane holds RPL consecutive key rows of its column of S in registers.
+// Per token:  S <- decay * S;  u = beta * (v - S^T k);  S <- S + k u^T;
+// o = S^T q   (the read-out sees the token's own write).
+// q, k, decay of DR_TC tokens at a time are staged in LDS (rows past D are
+// staged as zero so the inner loops need no bounds).
+#define DR_TC 16
+template <int RPL, typename TC>
+__global__ __launch_bounds__(64) void delta_recurrent_kernel(
+    const float* __restrict__ qn, const float* __restrict__ kn,
+    const float* __restrict__ decay, const float* __restrict__ beta,
+    const TC* __restrict__ v, int64_t vs, float* __restrict__ state,
+    float* __restrict__ out, const int* __restrict__ cu,
+    const int* __restrict__ past, const int* __restrict__ slots, int H, int G,
+    int D, int Dv) {
+    constexpr int DP = RPL * 4;  // padded key size
+    __shared__ float sq[DR_TC][DP];
+    __shared__ float sk[DR_TC][DP];
+    __shared__ float sg[DR_TC][DP];
+    const int b = blockIdx.x, h = blockIdx.y;
+    const int lane = threadIdx.x;
+    const int col = blockIdx.z * 16 + (lane & 15), rg = lane >> 4;
+    const bool col_ok = col < Dv;
+    const int lo = cu[b], n = cu[b + 1] - lo;
+    if (n <= 0) return;
+    const int kvh = h / (H / G);
+    float* st = state + (((int64_t)slots[b] * H + h) * D) * Dv;
+    float S[RPL];
+    const bool fresh = past[b] == 0;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+        const int r = rg * RPL + i;
+        S[i] = (!fresh && col_ok && r < D) ? st[(int64_t)r * Dv + col] : 0.0f;
+    }
+    for (int c0 = 0; c0 < n; c0 += DR_TC) {
+        const int nc = min(DR_TC, n - c0);
+        __builtin_amdgcn_wave_barrier();
+        for (int i = lane; i < nc * DP; i += 64) {
+            const int tt = i / DP, r = i % DP;
+            const int t = lo + c0 + tt;
+            const bool ok = r < D;
+            sq[tt][r] = ok ? qn[((int64_t)t * G + kvh) * D + r] : 0.0f;
+            sk[tt][r] = ok ? kn[((int64_t)t * G + kvh) * D + r] : 0.0f;
+            sg[tt][r] = ok ? decay[((int64_t)t * H + h) * D + r] : 0.0f;
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+        for (int tt = 0; tt < nc; ++tt) {
+            const int t = lo + c0 + tt;
+            const float bt = beta[(int64_t)t * H + h];
+            const float vv = col_ok ? ldf(v, (int64_t)t * vs + (int64_t)h * Dv + col) : 0.0f;
+            const float* kq = &sk[tt][rg * RPL];
+            const float* gq = &sg[tt][rg * RPL];
+            const float* qq = &sq[tt][rg * RPL];
+            float dot = 0.0f;
+#pragma unroll
+            for (int i = 0; i < RPL; ++i) {
+                S[i] *= gq[i];
+                dot += S[i] * kq[i];
+            }
+            dot += __shfl_xor(dot, 16, WAVE);
+            dot += __shfl_xor(dot, 32, WAVE);
+            const float u = bt * (vv - dot);
+            float o = 0.0f;
+#pragma unroll
+            for (int i = 0; i < RPL; ++i) {
+                S[i] += kq[i] * u;
+                o += S[i] * qq[i];
+            }
+            o += __shfl_xor(o, 16, WAVE);
+            o += __shfl_xor(o, 32, WAVE);
+            if (rg == 0 && col_ok) out[((int64_t)t * H + h) * Dv + col] = o;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+        const int r = rg * RPL + i;
+        if (col_ok && r < D) st[(int64_t)r * Dv + col] = S[i];
+    }
+}
+
+// per-head RMS norm of the read-out, times w[Dv], times sigmoid(gate):
+// one block per token, one wave per head
+template <typename TC>
+__global__ __launch_bounds__(256) void gated_head_norm_kernel(
+    const float* __restrict__ o, const TC* __restrict__ w,
+    const TC* __restrict__ gate, int64_t gs, TC* __restrict__ out, int H, int Dv,
+    float eps) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    for (int h = wave; h < H; h += nw) {
+        const float* src = o + ((int64_t)t * H + h) * Dv;
+        float ss = 0.0f;
+        for (int i = lane; i < Dv; i += 64) ss += src[i] * src[i];
+        ss = wave_reduce_sum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
+        for (int i = lane; i < Dv; i += 64) {
+            const float gt = sigmoidf_(ldf(gate, (int64_t)t * gs + h * Dv + i));
+            stf(out, ((int64_t)t * H + h) * Dv + i, src[i] * r * ldf(w, i) * gt);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// logits -> cap * tanh(logits / cap), float32 out
+template <typename TC>
+__global__ __launch_bounds__(256) void softcap_kernel(const TC* __restrict__ x,
+                                                      float* __restrict__ out,
+                                                      int64_t n, float cap) {
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x)
+        out[i] = cap * tanhf(ldf(x, i) / cap);
+}
+
+// silu(gate) * up over rows of a [M, 2I] gate|up buffer (any float type)
+template <typename TC>
+__global__ __launch_bounds__(256) void silu_mul_rows_kernel(const TC* __restrict__ gu,
+                                                            TC* __restrict__ out,
+                                                            int64_t M, int I) {
+    const int64_t total = M * I;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t m = idx / I;
+        const int i = (int)(idx % I);
+        const float g = ldf(gu, m * 2 * I + i), u = ldf(gu, m * 2 * I + I + i);
+        stf(out, idx, g * sigmoidf_(g) * u);
+    }
+}
+
+// float32 rows -> activation type (embedding rows gathered into the residual)
+template <typename TC>
+__global__ __launch_bounds__(256) void embed_rows_kernel(const TC* __restrict__ table,
+                                                         const int64_t* __restrict__ ids,
+                                                         float* __restrict__ out, int T,
+                                                         int C) {
+    const int64_t total = (int64_t)T * C;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int t = (int)(idx / C), c = (int)(idx % C);
+        out[idx] = ldf(table, ids[t] * (int64_t)C + c);
+    }
+}
+
+// ===========================================================================
+// C entry points. dt: 0 = bf16 activations/weights, 1 = float32.
+static inline int grid_for(int64_t total) {
+    return (int)std::max<int64_t>(1, std::min<int64_t>(4096, CEIL_DIV(total, 256)));
+}
+
+// x_dt: type of x (0 bf16, 1 f32); dt: type of w and out
+extern "C" int oa_causal_conv_seq(void* stream, const void* x, int64_t xs, int x_dt,
+                                  const void* w, void* state, void* out, int64_t os,
+                                  const void* seq_of, const void* cu, const void* past,
+                                  const void* slots, int T, int B, int C, int taps,
+                                  int add_input, int act_silu, int dt) {
+    if (T <= 0) return 0;
+    if (taps < 1) return -100;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 g1(grid_for((int64_t)T * C)), g2(grid_for((int64_t)B * C)), blk(256);
+#define CONV_ARGS(TI, TW)                                                          \
+    (const TI*)x, xs, (const TW*)w, (const float*)state, (TW*)out, os,             \
+        (const int*)seq_of, (const int*)cu, (const int*)past, (const int*)slots, T, \
+        C, taps, add_input, act_silu
+    if (x_dt == 1 && dt == 1)
+        hipLaunchKernelGGL((causal_conv_kernel<float, float, float>), g1, blk, 0, s, CONV_ARGS(float, float));
+    else if (x_dt == 1 && dt == 0)
+        hipLaunchKernelGGL((causal_conv_kernel<float, bf16s, bf16s>), g1, blk, 0, s, CONV_ARGS(float, bf16s));
+    else if (x_dt == 0 && dt == 0)
+        hipLaunchKernelGGL((causal_conv_kernel<bf16s, bf16s, bf16s>), g1, blk, 0, s, CONV_ARGS(bf16s, bf16s));
+    else
+        return -101;
+#undef CONV_ARGS
+    HIP_CHECK_LAUNCH();
+    if (taps > 1) {
+        if (x_dt == 1)
+            hipLaunchKernelGGL((conv_state_update_kernel<float>), g2, blk, 0, s, (const float*)x, xs,
+                               (float*)state, (const int*)cu, (const int*)past, (const int*)slots, B, C, taps);
+        else
+            hipLaunchKernelGGL((conv_state_update_kernel<bf16s>), g2, blk, 0, s, (const bf16s*)x, xs,
+                               (float*)state, (const int*)cu, (const int*)past, (const int*)slots, B, C, taps);
+        HIP_CHECK_LAUNCH();
+    }
+    return 0;
+}
+
+// y_dt: type of y; dt: type of w and copy. residual/copy may be null (not both).
+extern "C" int oa_group_rmsnorm(void* stream, const void* y, int64_t ys, int y_dt,
+                                const void* w, void* residual, void* copy, int T, int C,
+                                int groups, float eps, int dt) {
+    if (T <= 0) return 0;
+    if (groups < 1 || C % groups != 0 || (!residual && !copy)) return -100;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 g(T), blk(256);
+#define GN_ARGS(TY, TW) (const TY*)y, ys, (const TW*)w, (float*)residual, (TW*)copy, C, groups, eps
+    if (y_dt == 1 && dt == 1)
+        hipLaunchKernelGGL((group_rmsnorm_kernel<float, float, float>), g, blk, 0, s, GN_ARGS(float, float));
+    else if (y_dt == 1 && dt == 0)
+        hipLaunchKernelGGL((group_rmsnorm_kernel<float, bf16s, bf16s>), g, blk, 0, s, GN_ARGS(float, bf16s));
+    else if (y_dt == 0 && dt == 0)
+        hipLaunchKernelGGL((group_rmsnorm_kernel<bf16s, bf16s, bf16s>), g, blk, 0, s, GN_ARGS(bf16s, bf16s));
+    else
+        return -101;
+#undef GN_ARGS
+    HIP_CHECK_LAUNCH();
+    return 0;
+}
+
+extern "C" int oa_attn_prepare(void* stream, const void* qkv, int64_t qs, const void* bias, const void* qw,
+                               const void* kw, void* q_out, void* k_cache, void* v_cache,
+                               const void* slot_mapping, const void* cu, int B, int T, int H,
+                               int G, int D, int Dv, float eps, int dt) {
+    if (T <= 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dt == 1)
+        hipLaunchKernelGGL((attn_prepare_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)qkv, qs,
+                           (const float*)bias, (const float*)qw, (const float*)kw, (float*)q_out, (float*)k_cache,
+                           (float*)v_cache, (const int*)slot_mapping, (const int*)cu, B, H, G, D, Dv, eps);
+    else
+        hipLaunchKernelGGL((attn_prepare_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const bf16s*)qkv, qs,
+                           (const bf16s*)bias, (const bf16s*)qw, (const bf16s*)kw, (bf16s*)q_out, (bf16s*)k_cache,
+                           (bf16s*)v_cache, (const int*)slot_mapping, (const int*)cu, B, H, G, D, Dv, eps);
+    HIP_CHECK_LAUNCH();
+    return 0;
+}
+
+// Geometry the host must agree with: tile size, key-tile size, LDS bytes.
+extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int* TQ, int* KT,
+                                     int* kstride, int* lds_bytes) {
+    if (G < 1 || H % G != 0 || Dv > 64 * ATT_MAXV) return -100;
+    const int R = H / G;
+    if (R > 4 * ATT_MAXR) return -102;
+    int tq = std::max(1, (4 * ATT_MAXR) / R);
+    const int esz = dt == 1 ? 4 : 2;
+    int ks = D;
+    if (dt == 1) ks = (D % 2 == 0) ? D + 1 : D;
+    else ks = ((D / 2) % 2 == 0) ? D + 2 : D + (D % 2);
+    for (int kt = 64; kt >= 8; kt >>= 1) {
+        size_t bytes = ((size_t)tq * R * D + 4 * kt) * 4 + ((size_t)kt * ks + (size_t)kt * Dv) * esz;
+        if (bytes <= 64 * 1024) {
+            *TQ = tq; *KT = kt; *kstride = ks; *lds_bytes = (int)bytes;
+            return 0;
+        }
+    }
+    return -103;
+}
+
+// ntiles = sum_b ceil(n_b / TQ) (host-computed). part_* may be null when nsplit == 1.
+extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate, int64_t gs,
+                                  const void* k_cache, const void* v_cache, void* out,
+                                  void* part_o, void* part_ml, const void* cu, const void* past,
+                                  const void* block_table, int max_blocks, int block_size,
+                                  const void* slopes, int T, int B, int ntiles, int H, int G,
+                                  int D, int Dv, float scale, int nsplit, int dt) {
+    if (T <= 0 || ntiles <= 0) return 0;
+    int TQ, KT, ks, lds_bytes;
+    int rc = oa_attn_bias_geometry(H, G, D, Dv, dt, &TQ, &KT, &ks, &lds_bytes);
+    if (rc) return rc;
+    if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return -104;
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(ntiles, G, nsplit), blk(256);
+#define AT_ARGS(TC)                                                                      \
+    (const TC*)q, (const TC*)gate, gs, (const TC*)k_cache, (const TC*)v_cache, (TC*)out,  \
+        (float*)part_o, (float*)part_ml, (const int*)cu, (const int*)past,                \
+        (const int*)block_table, max_blocks, block_size, (const float*)slopes, B, H, G, D, \
+        Dv, TQ, KT, ks, scale, nsplit
+    if (dt == 1)
+        hipLaunchKernelGGL((attn_bias_paged_kernel<float>), grid, blk, lds_bytes, s, AT_ARGS(float));
+    else
+        hipLaunchKernelGGL((attn_bias_paged_kernel<bf16s>), grid, blk, lds_bytes, s, AT_ARGS(bf16s));
+#undef AT_ARGS
+    HIP_CHECK_LAUNCH();
+    if (nsplit > 1) {
+        if (dt == 1)
+            hipLaunchKernelGGL((attn_combine_kernel<float>), dim3((unsigned)((int64_t)T * H)), dim3(64), 0, s,
+                               (const float*)part_o, (const float*)part_ml, (const float*)gate, gs,
+                               (float*)out, H, Dv, nsplit);
+        else
+            hipLaunchKernelGGL((attn_combine_kernel<bf16s>), dim3((unsigned)((int64_t)T * H)), dim3(64), 0, s,
+                               (const float*)part_o, (const float*)part_ml, (const bf16s*)gate, gs,
+                               (bf16s*)out, H, Dv, nsplit);
+        HIP_CHECK_LAUNCH();
+    }
+    return 0;
+}
+
+extern "C" int oa_delta_prepare(void* stream, const void* q, int64_t qs, const void* k, int64_t ks,
+                                const void* bl, int64_t bs, const void* a, int64_t as,
+                                const void* dt_bias, const void* a_log, void* qn, void* kn,
+                                void* decay, void* beta, int T, int H, int G, int D, int dt) {
+    if (T <= 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dt == 1)
+        hipLaunchKernelGGL((delta_prepare_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)q, qs,
+                           (const float*)k, ks, (const float*)bl, bs, (const float*)a, as,
+                           (const float*)dt_bias, (const float*)a_log, (float*)qn, (float*)kn,
+                           (float*)decay, (float*)beta, H, G, D);
+    else
+        hipLaunchKernelGGL((delta_prepare_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const bf16s*)q, qs,
+                           (const bf16s*)k, ks, (const bf16s*)bl, bs, (const bf16s*)a, as,
+                           (const bf16s*)dt_bias, (const bf16s*)a_log, (float*)qn, (float*)kn,
+                           (float*)decay, (float*)beta, H, G, D);
+    HIP_CHECK_LAUNCH();
+    return 0;
+}
+
+template <int RPL>
+static int launch_delta(hipStream_t s, const void* qn, const void* kn, const void* decay,
+                        const void* beta, const void* v, int64_t vs, void* state, void* out,
+                        const void* cu, const void* past, const void* slots, int B, int H,
+                        int G, int D, int Dv, int dt) {
+    dim3 grid(B, H, CEIL_DIV(Dv, 16)), blk(64);
+    if (dt == 1)
+        hipLaunchKernelGGL((delta_recurrent_kernel<RPL, float>), grid, blk, 0, s, (const float*)qn,
+                           (const float*)kn, (const float*)decay, (const float*)beta, (const float*)v,
+                           vs, (float*)state, (float*)out, (const int*)cu, (const int*)past,
+                           (const int*)slots, H, G, D, Dv);
+    else
+        hipLaunchKernelGGL((delta_recurrent_kernel<RPL, bf16s>), grid, blk, 0, s, (const float*)qn,
+                           (const float*)kn, (const float*)decay, (const float*)beta, (const bf16s*)v,
+                           vs, (float*)state, (float*)out, (const int*)cu, (const int*)past,
+                           (const int*)slots, H, G, D, Dv);
+    HIP_CHECK_LAUNCH();
+    return 0;
+}
+
+extern "C" int oa_delta_recurrent(void* stream, const void* qn, const void* kn, const void* decay,
+                                  const void* beta, const void* v, int64_t vs, void* state,
+                                  void* out, const void* cu, const void* past, const void* slots,
+                                  int T, int B, int H, int G, int D, int Dv, int dt) {
+    if (T <= 0 || B <= 0) return 0;
+    if (G < 1 || H % G != 0) return -100;
+    hipStream_t s = (hipStream_t)stream;
+#define DL(R) launch_delta<R>(s, qn, kn, decay, beta, v, vs, state, out, cu, past, slots, B, H, G, D, Dv, dt)
+    if (D <= 32) return DL(8);
+    if (D <= 64) return DL(16);
+    if (D <= 96) return DL(24);
+    if (D <= 128) return DL(32);
+    if (D <= 192) return DL(48);
+    if (D <= 256) return DL(64);
+#undef DL
+    return -105;
+}
+
+extern "C" int oa_gated_head_norm(void* stream, const void* o, const void* w, const void* gate,
+                                  int64_t gs, void* out, int T, int H, int Dv, float eps, int dt) {
+    if (T <= 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dt == 1)
+        hipLaunchKernelGGL((gated_head_norm_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)o,
+                           (const float*)w, (const float*)gate, gs, (float*)out, H, Dv, eps);
+    else
+        hipLaunchKernelGGL((gated_head_norm_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const float*)o,
+                           (const bf16s*)w, (const bf16s*)gate, gs, (bf16s*)out, H, Dv, eps);
+    HIP_CHECK_LAUNCH();
+    return 0;
+}
+
+extern "C" int oa_softcap(void* stream, const void* x, void* out, int64_t n, float cap, int dt) {
+    if (n <= 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dt == 1)
+        hipLaunchKernelGGL((softcap_kernel<float>), dim3(grid_for(n)), dim3(256), 0, s, (const float*)x,
+                           (float*)out, n, cap);
+    else
+        hipLaunchKernelGGL((softcap_kernel<bf16s>), dim3(grid_for(n)), dim3(256), 0, s, (const bf16s*)x,
+                           (float*)out, n, cap);
+    HIP_CHECK_LAUNCH();
+    return 0;
+}
+
+extern "C" int oa_silu_mul_rows(void* stream, const void* gu, void* out, int64_t M, int I, int dt) {
+    if (M <= 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dt == 1)
+        hipLaunchKernelGGL((silu_mul_rows_kernel<float>), dim3(grid_for(M * I)), dim3(256), 0, s,
+                           (const float*)gu, (float*)out, M, I);
+    else
+        hipLaunchKernelGGL((silu_mul_rows_kernel<bf16s>), dim3(grid_for(M * I)), dim3(256), 0, s,
+                           (const bf16s*)gu, (bf16s*)out, M, I);
+    HIP_CHECK_LAUNCH();
+    return 0;
+}
+
+extern "C" int oa_embed_rows(void* stream, const void* table, const void* ids, void* out, int T,
+                             int C, int dt) {
+    if (T <= 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (dt == 1)
+        hipLaunchKernelGGL((embed_rows_kernel<float>), dim3(grid_for((int64_t)T * C)), dim3(256), 0, s,
+                           (const float*)table, (const int64_t*)ids, (float*)out, T, C);
+    else
+        hipLaunchKernelGGL((embed_rows_kernel<bf16s>), dim3(grid_for((int64_t)T * C)), dim3(256), 0, s,
+                           (const bf16s*)table, (const int64_t*)ids, (float*)out, T, C);
+    HIP_CHECK_LAUNCH();
+    return 0;
+}

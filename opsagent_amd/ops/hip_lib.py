@@ -103,6 +103,58 @@ def get_lib() -> ctypes.CDLL:
     return _LIB
 
 
+_MIXERS: Optional[ctypes.CDLL] = None
+_MIXERS_PATH = os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "libopsagent_mixers.so"
+)
+
+
+def _declare_mixers(lib: ctypes.CDLL) -> None:
+    p = ctypes.c_void_p
+    i = ctypes.c_int
+    i64 = ctypes.c_int64
+    f = ctypes.c_float
+    ip = ctypes.POINTER(ctypes.c_int)
+    sigs = {
+        "oa_causal_conv_seq": [p, p, i64, i, p, p, p, i64, p, p, p, p, i, i, i, i, i, i, i],
+        "oa_group_rmsnorm": [p, p, i64, i, p, p, p, i, i, i, f, i],
+        "oa_attn_prepare": [p, p, i64, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i],
+        "oa_attn_bias_geometry": [i, i, i, i, i, ip, ip, ip, ip],
+        "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p,
+                               i, i, i, i, i, i, i, f, i, i],
+        "oa_delta_prepare": [p, p, i64, p, i64, p, i64, p, i64, p, p, p, p, p, p,
+                             i, i, i, i, i],
+        "oa_delta_recurrent": [p, p, p, p, p, p, i64, p, p, p, p, p, i, i, i, i, i, i, i],
+        "oa_gated_head_norm": [p, p, p, p, i64, p, i, i, i, f, i],
+        "oa_softcap": [p, p, p, i64, f, i],
+        "oa_silu_mul_rows": [p, p, p, i64, i, i],
+        "oa_embed_rows": [p, p, p, p, i, i, i],
+    }
+    for name, args in sigs.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = i
+
+
+def get_mixers_lib() -> ctypes.CDLL:
+    """The sequence-mixer kernel library (hybrid decoders); built in-tree on
+    first use if the checkout has no built copy."""
+    global _MIXERS
+    if _MIXERS is None:
+        try:
+            from opsagent_amd.ops.build import build_mixers
+
+            build_mixers(verbose=False)
+        except Exception as e:
+            if not os.path.exists(_MIXERS_PATH):
+                raise HipKernelsMissing(
+                    f"mixer kernel library missing and build failed: {e}"
+                ) from e
+        _MIXERS = ctypes.CDLL(_MIXERS_PATH)
+        _declare_mixers(_MIXERS)
+    return _MIXERS
+
+
 def available() -> bool:
     try:
         get_lib()

@@ -177,3 +177,156 @@ def greedy_sample_masked(logits: torch.Tensor, mask: Optional[torch.Tensor]) -> 
     if mask is not None:
         lf = lf.masked_fill(~mask, float("-inf"))
     return lf.argmax(dim=-1)
+
+
+# ---------------------------------------------------------------------------
+# Sequence-mixer ops over a flat multi-sequence batch (CPU path and numerics
+# reference of mixers.hip). A batch is T tokens of B sequences laid end to
+# end: cu[b]..cu[b+1] are sequence b's new tokens, which continue it from
+# position past[b]; slots[b] is its row in the state tensors.
+
+
+def causal_conv_seq(x, w, state, cu, past, slots, add_input, act_silu, out_dtype):
+    """Causal per-channel convolution over time, continued from `state`
+    (the last taps-1 inputs of each sequence, float32 [slots, taps-1, C]);
+    inputs before position 0 are zero whatever the slot holds. Returns
+    (x if add_input) + conv(x), optionally through silu; updates state."""
+    taps = w.shape[1]
+    wf = w.float()
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        xs = x[lo:hi].float()
+        if taps > 1:
+            prev = state[slots[b]].clone()
+            keep = min(past[b], taps - 1)
+            prev[: taps - 1 - keep] = 0
+            ext = torch.cat([prev, xs], 0)
+        else:
+            ext = xs
+        n = hi - lo
+        y = torch.zeros_like(xs)
+        for j in range(taps):
+            y += ext[j : j + n] * wf[:, j]
+        if add_input:
+            y += xs
+        if act_silu:
+            y = torch.nn.functional.silu(y)
+        out[lo:hi] = y.to(out_dtype)
+        if taps > 1:
+            state[slots[b]] = ext[-(taps - 1):]
+    return out
+
+
+def group_rms_norm(y, w, groups, eps, residual, out_dtype):
+    """RMS norm over `groups` equal consecutive parts of the last axis, times
+    w. With `residual` (float32, updated in place) returns residual + norm."""
+    T, C = y.shape
+    yf = y.float().view(T, groups, C // groups)
+    n = (yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps)).view(T, C) * w.float()
+    if residual is not None:
+        residual += n
+        return residual
+    return n.to(out_dtype)
+
+
+def attn_qkv_prepare(qkv, bias, q_norm_w, k_norm_w, H, G, D, Dv, eps, k_cache, v_cache,
+                     slot_mapping):
+    """Adds the projection bias (if any), then whole-projection RMS norm of q
+    and of k (weighted), per-head RMS norm of v (no weight); k and v go to
+    their cache slots, q is returned."""
+    T = qkv.shape[0]
+    n = H * D + G * D + G * Dv
+    x = qkv[:, :n].float()
+    if bias is not None:
+        x = x + bias[:n].float()
+    q, k, v = x[:, : H * D], x[:, H * D : H * D + G * D], x[:, H * D + G * D :]
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm_w.float()
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm_w.float()
+    v = v.reshape(T, G, Dv)
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    nb, bs = k_cache.shape[0], k_cache.shape[1]
+    sm = slot_mapping.long()
+    k_cache.view(nb * bs, G, D)[sm] = k.reshape(T, G, D).to(k_cache.dtype)
+    v_cache.view(nb * bs, G, Dv)[sm] = v.to(v_cache.dtype)
+    return q.reshape(T, H, D).to(qkv.dtype)
+
+
+def attention_biased_paged(q, gate_logits, k_cache, v_cache, cu, past, block_table,
+                           scale, slopes):
+    """Causal softmax attention of each new token over its sequence's cached
+    keys 0..position, score = q.k*scale - slope_h*(i-j), each head's output
+    times sigmoid(gate logit). q [T,H,D]; returns [T, H*Dv]."""
+    T, H, D = q.shape
+    nb, bs, G, Dv = v_cache.shape
+    out = torch.empty(T, H, Dv, dtype=q.dtype, device=q.device)
+    rep = H // G
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        total = past[b] + hi - lo
+        nblk = (total + bs - 1) // bs
+        blocks = block_table[b, :nblk].long()
+        kk = k_cache[blocks].reshape(nblk * bs, G, D)[:total].float()
+        vv = v_cache[blocks].reshape(nblk * bs, G, Dv)[:total].float()
+        kk = kk.repeat_interleave(rep, dim=1)
+        vv = vv.repeat_interleave(rep, dim=1)
+        qs = q[lo:hi].float()
+        s = torch.einsum("ihd,jhd->hij", qs, kk) * scale
+        i = torch.arange(past[b], total, dtype=torch.float32).view(1, -1, 1)
+        j = torch.arange(total, dtype=torch.float32).view(1, 1, -1)
+        s = s - slopes.float().view(H, 1, 1) * (i - j)
+        s = s.masked_fill(j > i, float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        o = torch.einsum("hij,jhd->ihd", p, vv)
+        o = o * torch.sigmoid(gate_logits[lo:hi].float()).unsqueeze(-1)
+        out[lo:hi] = o.to(q.dtype)
+    return out.view(T, H * Dv)
+
+
+def channel_delta_rule(q, k, v, b_logits, a, dt_bias, a_log, state, cu, past, slots):
+    """Gated delta rule with a decay per head and key channel, continued from
+    `state` [slots, H, D, Dv] float32 (zero at position 0 whatever the slot
+    holds). q,k [T,G,D], v [T,H,Dv] after convolution and silu; b_logits
+    [T,H]; a [T,H*D]. Returns the read-out [T,H,Dv] float32; updates state."""
+    T, G, D = q.shape
+    H, Dv = v.shape[1], v.shape[2]
+    rep = H // G
+    qf, kf = q.float(), k.float()
+    qf = qf * torch.rsqrt(qf.pow(2).sum(-1, keepdim=True) + 1e-6) * (D ** -0.5)
+    kf = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + 1e-6)
+    qf = qf.repeat_interleave(rep, dim=1)
+    kf = kf.repeat_interleave(rep, dim=1)
+    beta = torch.sigmoid(b_logits.float())
+    sp = torch.nn.functional.softplus(a.float() + dt_bias.float())
+    g = torch.exp(-torch.exp(a_log.float()).view(1, H, 1) * sp.view(T, H, D))
+    vf = v.float()
+    out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
+    for bi in range(len(cu) - 1):
+        lo, hi = cu[bi], cu[bi + 1]
+        if hi == lo:
+            continue
+        S = state[slots[bi]].clone() if past[bi] > 0 else torch.zeros_like(state[slots[bi]])
+        for t in range(lo, hi):
+            S = S * g[t].unsqueeze(-1)
+            u = beta[t].unsqueeze(-1) * (vf[t] - torch.einsum("hdv,hd->hv", S, kf[t]))
+            S = S + kf[t].unsqueeze(-1) * u.unsqueeze(1)
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slots[bi]] = S
+    return out
+
+
+def gated_head_rms_norm(o, w, gate_logits, eps, out_dtype):
+    """o [T,H,Dv] float32: per-head RMS norm, times w [Dv], times
+    sigmoid(gate_logits [T, H*Dv]). Returns [T, H*Dv]."""
+    T, H, Dv = o.shape
+    n = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    n = n * torch.sigmoid(gate_logits.float()).view(T, H, Dv)
+    return n.reshape(T, H * Dv).to(out_dtype)
+
+
+def softcap(logits, cap):
+    return cap * torch.tanh(logits.float() / cap)
