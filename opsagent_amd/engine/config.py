@@ -356,13 +356,19 @@ def load_spec_from_dir(path: str):
     spec = ARCHITECTURE_PARSERS[arch](cfg, name=os.path.basename(os.path.normpath(path)))
     spec.weights_path = os.path.join(path, "model.safetensors")
     if os.path.exists(spec.weights_path):
-        shapes = safetensors_shapes(spec.weights_path)
-        for i, layer in enumerate(spec.layers):
-            a1, g1 = shapes.get(f"l{i}.mix.a1"), shapes.get(f"l{i}.mix.g1")
-            if a1 is not None:
-                layer.mixer.decay_rank = int(a1[0])
-            if g1 is not None:
-                layer.mixer.gate_rank = int(g1[0])
+        apply_tensor_shapes(spec, safetensors_shapes(spec.weights_path))
+    return spec
+
+
+def apply_tensor_shapes(spec: HybridSpec, shapes: dict) -> HybridSpec:
+    """Fill the sizes that only tensor shapes give (name -> shape): the inner
+    ranks of the low-rank decay and output-gate projections."""
+    for i, layer in enumerate(spec.layers):
+        a1, g1 = shapes.get(f"l{i}.mix.a1"), shapes.get(f"l{i}.mix.g1")
+        if a1 is not None:
+            layer.mixer.decay_rank = int(a1[0])
+        if g1 is not None:
+            layer.mixer.gate_rank = int(g1[0])
     return spec
 
 

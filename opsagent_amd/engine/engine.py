@@ -285,6 +285,12 @@ class LLMEngine:
         self._prefer_decode = False
         self.perf = get_perf_stats()
         self._graphs: Dict[int, Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        pin = self.device == "cuda"
+        words_pin = (self.spec.vocab_size + 31) // 32
+        self._h_mask = torch.empty(
+            self.max_batch, words_pin, dtype=torch.int32, pin_memory=pin
+        )
+        self._h_ones = torch.full((words_pin,), -1, dtype=torch.int32)
         if self.hybrid:
             # per-layer cache geometry comes from the model's mixers; every
             # live sequence also owns one slot of recurrent/convolution state
@@ -319,11 +325,6 @@ class LLMEngine:
         self._h_pos = torch.empty(self.max_batch, dtype=torch.int32, pin_memory=pin)
         self._h_slots = torch.empty(self.max_batch, dtype=torch.int32, pin_memory=pin)
         self._h_lens = torch.empty(self.max_batch, dtype=torch.int32, pin_memory=pin)
-        words_pin = (self.spec.vocab_size + 31) // 32
-        self._h_mask = torch.empty(
-            self.max_batch, words_pin, dtype=torch.int32, pin_memory=pin
-        )
-        self._h_ones = torch.full((words_pin,), -1, dtype=torch.int32)
         self._dec_input = torch.zeros(self.max_batch, dtype=torch.int64, device=dev)
         self._dec_pos = torch.zeros(self.max_batch, dtype=torch.int32, device=dev)
         self._dec_slots = torch.zeros(self.max_batch, dtype=torch.int32, device=dev)

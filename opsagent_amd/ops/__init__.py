@@ -761,10 +761,22 @@ def greedy_sample_masked(
     [B, ceil(V/32)] on GPU, bool [B, V] on CPU. Returns int32/int64 [B]."""
     if not _is_gpu(logits):
         return torch_ref.greedy_sample_masked(logits, mask_bits)
-    assert logits.dtype == torch.bfloat16 and logits.is_contiguous()
     lib, hip = _lib()
     B, V = logits.shape
     out = torch.empty(B, dtype=torch.int32, device=logits.device)
+    if logits.dtype == torch.float32:
+        # float32 rows of any width (hybrid models' soft-capped logits)
+        assert logits.is_contiguous()
+        if mask_bits is not None:
+            assert mask_bits.dtype == torch.int32 and mask_bits.is_contiguous()
+        rc = lib.oa_masked_argmax_f32(
+            hip.current_stream_ptr(), logits.data_ptr(),
+            mask_bits.data_ptr() if mask_bits is not None else None,
+            out.data_ptr(), B, V,
+        )
+        hip.check(rc, "oa_masked_argmax_f32")
+        return out
+    assert logits.dtype == torch.bfloat16 and logits.is_contiguous()
     ws = torch.empty(B, dtype=torch.int64, device=logits.device)
     mask_ptr = mask_bits.data_ptr() if mask_bits is not None else None
     if mask_bits is not None:

@@ -118,3 +118,58 @@ extern "C" int oa_masked_argmax(void* stream, const void* logits, const void* ma
     HIP_CHECK_LAUNCH();
     return 0;
 }
+
+// float32 logits (models whose head emits float32, any V): one block per
+// row scans the whole row; lowest index wins ties, -1 if nothing is allowed.
+__global__ __launch_bounds__(256) void masked_argmax_f32_kernel(
+    const float* __restrict__ logits, const uint32_t* __restrict__ mask,
+    int* __restrict__ out, int V, int mask_words) {
+    const int b = blockIdx.x;
+    const float* row = logits + (size_t)b * V;
+    const uint32_t* mrow = mask ? mask + (size_t)b * mask_words : nullptr;
+    float best = -INFINITY;
+    int besti = -1;
+    for (int t = threadIdx.x; t < V; t += blockDim.x) {
+        if (mrow && !((mrow[t >> 5] >> (t & 31)) & 1u)) continue;
+        const float v = row[t];
+        if (besti < 0 || v > best) {  // ascending t per thread: first max kept
+            best = v;
+            besti = t;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        float ov = __shfl_xor(best, off, WAVE);
+        int oi = __shfl_xor(besti, off, WAVE);
+        if (oi >= 0 && (besti < 0 || ov > best || (ov == best && oi < besti))) {
+            best = ov;
+            besti = oi;
+        }
+    }
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const int wid = threadIdx.x / WAVE;
+    if ((threadIdx.x & (WAVE - 1)) == 0) {
+        sv[wid] = best;
+        si[wid] = besti;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (si[w] >= 0 && (besti < 0 || sv[w] > best || (sv[w] == best && si[w] < besti))) {
+                best = sv[w];
+                besti = si[w];
+            }
+        out[b] = besti;
+    }
+}
+
+extern "C" int oa_masked_argmax_f32(void* stream, const void* logits, const void* mask,
+                                    void* out, int B, int V) {
+    if (B <= 0) return 0;
+    hipLaunchKernelGGL(masked_argmax_f32_kernel, dim3(B), dim3(256), 0,
+                       (hipStream_t)stream, (const float*)logits, (const uint32_t*)mask,
+                       (int*)out, V, CEIL_DIV(V, 32));
+    HIP_CHECK_LAUNCH();
+    return 0;
+}

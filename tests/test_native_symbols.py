@@ -21,7 +21,7 @@ ENTRY_POINTS = [
     "oa_gemv", "oa_gemv_bf16_mfma", "oa_gemv_ex", "oa_gemv_fp8",
     "oa_gemv_fp8_ex", "oa_gemv_fp8_mfma", "oa_gemv_gateup",
     "oa_gemv_gateup_ex", "oa_gemv_gateup_fp8", "oa_gemv_rw4", "oa_kv_write",
-    "oa_masked_argmax", "oa_moe_down", "oa_moe_down_emaj", "oa_moe_gateup",
+    "oa_masked_argmax", "oa_masked_argmax_f32", "oa_moe_down", "oa_moe_down_emaj", "oa_moe_gateup",
     "oa_moe_gateup_emaj", "oa_quant_fp8", "oa_rmsnorm", "oa_rope",
     "oa_rope_kv", "oa_silu_mul",
 ]
