@@ -80,7 +80,15 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=8)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--model", default="llama3-8b")
-    ap.add_argument("--mode", choices=["turn", "multiturn", "concurrent"], default="turn")
+    ap.add_argument("--mode", choices=["turn", "multiturn", "concurrent", "layers"],
+                    default="turn",
+                    help="layers: prefill/decode throughput of the Povazen hybrid "
+                         "decoder beside llama layers of equal size (extra mode; "
+                         "prints one JSON line per size and batch)")
+    ap.add_argument("--layer-models", default="llama,povazen",
+                    help="layers mode: which models to run")
+    ap.add_argument("--layer-sizes", default="", help="layers mode: size names (default all)")
+    ap.add_argument("--layer-batches", default="1,8", help="layers mode: batch sizes")
     ap.add_argument("--concurrency", type=int, default=8, help="sessions in concurrent mode")
     ap.add_argument("--moe-dtype", default=None, help="fp8 to quantize MoE experts")
     ap.add_argument("--decode-tokens", type=int, default=128)
@@ -96,6 +104,19 @@ def main() -> None:
                          "(trained BPE, scripts/train_tokenizer.py), "
                          "'byte' = byte-level, or a tokenizer.json path")
     args = ap.parse_args()
+
+    if args.mode == "layers":
+        from opsagent_amd.utils import layer_bench
+
+        sizes = [z for z in layer_bench.SIZES
+                 if not args.layer_sizes or z[0] in args.layer_sizes.split(",")]
+        for row in layer_bench.run(sizes=sizes,
+                                   batches=tuple(int(b) for b in args.layer_batches.split(",")),
+                                   prompt=args.prompt_tokens if args.prompt_tokens != 1024 else 2048,
+                                   decode=max(8, min(args.decode_tokens, 64)),
+                                   models=tuple(args.layer_models.split(","))):
+            print(json.dumps(row), flush=True)
+        return
 
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -19,6 +19,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 typedef uint16_t bf16s;  // bf16 storage
 
@@ -337,6 +338,200 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same attention on the matrix cores (bf16 activations, key and value
+// sizes multiples of 16). Each wave owns 16 consecutive new tokens of one
+// query head; the 4 waves of a block are HB heads of one kv head times 4/HB
+// token sub-tiles, and share the staged key/value tiles.
+//
+// Swapped products keep everything in registers: S^T = K Q^T puts a token in
+// a lane's column (lane & 15), so the online-softmax statistics are per-lane
+// scalars, and S^T's accumulator layout IS the B-operand layout of
+// O^T = V^T P^T. v_mfma_f32_16x16x16_bf16: A[i][k]: lane holds i = lane&15,
+// k = 4*(lane>>4)..+3; B[k][j]: j = lane&15, same k; C[i][j]: j = lane&15,
+// i = 4*(lane>>4)..+3.
+// Scores, the distance penalty, softmax statistics and weights are float32;
+// a weight enters the value product as a bf16 pair hi + lo (two MFMAs), so
+// it keeps 16 bits of mantissa.
+// LDS: K tile [64][D+4], V tile transposed [Dv][64+4] (bf16).
+typedef short s4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+#define MF_KT 64
+
+template <int MAXD, int MAXDV>
+__global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
+    const bf16s* __restrict__ q, const bf16s* __restrict__ gate, int64_t gs,
+    const bf16s* __restrict__ k_cache, const bf16s* __restrict__ v_cache,
+    bf16s* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int* __restrict__ cu, const int* __restrict__ past,
+    const int* __restrict__ block_table, int max_blocks, int block_size,
+    const float* __restrict__ slopes, int B, int H, int G, int D, int Dv, int HB,
+    float scale, int nsplit) {
+    extern __shared__ float lds[];
+    bf16s* Ks = (bf16s*)lds;                        // [64][D+4]
+    const int kst = D + 4;
+    bf16s* Vt = Ks + (size_t)MF_KT * kst;           // [Dv][68]
+    const int vst = MF_KT + 4;
+    const int R = H / G;
+    const int TT = 4 / HB, TQ = 16 * TT;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lc = lane & 15, lg = lane >> 4;
+    const int hgroups = R / HB;
+    const int g = blockIdx.y / hgroups;
+    const int h = g * R + (blockIdx.y % hgroups) * HB + wave % HB;
+    const int split = blockIdx.z;
+    int tile = blockIdx.x, b = 0, lo = 0, n = 0;
+    for (; b < B; ++b) {
+        lo = cu[b];
+        n = cu[b + 1] - lo;
+        const int nt = (n + TQ - 1) / TQ;
+        if (tile < nt) break;
+        tile -= nt;
+    }
+    if (b >= B) return;
+    const int pb = past[b];
+    const int t0 = tile * TQ + (wave / HB) * 16;    // this wave's first local token
+    const int ntok = max(0, min(16, n - t0));
+    const int pos = pb + t0 + lc;                   // this lane's token position
+    const int wave_last = pb + t0 + ntok - 1;
+    const int block_last = pb + min(n, tile * TQ + TQ) - 1;
+    const int* bt = block_table + (int64_t)b * max_blocks;
+    const float slope = slopes[h];
+
+    s4_t qf[MAXD];
+    {
+        const int tk = lo + t0 + min(lc, max(ntok - 1, 0));
+        const bf16s* qr = q + ((int64_t)tk * H + h) * D + 4 * lg;
+#pragma unroll
+        for (int ks = 0; ks < MAXD; ++ks) {
+            if (16 * ks < D && ntok > 0) qf[ks] = *reinterpret_cast<const s4_t*>(qr + 16 * ks);
+            else qf[ks] = s4_t{0, 0, 0, 0};
+        }
+    }
+    f4_t o[MAXDV];
+#pragma unroll
+    for (int i = 0; i < MAXDV; ++i) o[i] = f4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.0f;
+
+    const int nkt = block_last / MF_KT + 1;
+    const int dch = D / 8, vch = Dv / 8;
+    for (int kt = split; kt < nkt; kt += nsplit) {
+        const int k0 = kt * MF_KT;
+        const int nk = min(MF_KT, block_last + 1 - k0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < MF_KT * dch; i += 256) {
+            const int j = i / dch, c = i % dch;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (j < nk) {
+                const int key = k0 + j;
+                const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
+                v = *reinterpret_cast<const uint4*>(k_cache + (slot * G + g) * D + 8 * c);
+            }
+            uint2* dst = reinterpret_cast<uint2*>(Ks + j * kst + 8 * c);
+            dst[0] = make_uint2(v.x, v.y);
+            dst[1] = make_uint2(v.z, v.w);
+        }
+        for (int i = threadIdx.x; i < MF_KT * vch; i += 256) {
+            const int j = i % MF_KT, c = i / MF_KT;   // lanes along keys: adjacent LDS columns
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (j < nk) {
+                const int key = k0 + j;
+                const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
+                v = *reinterpret_cast<const uint4*>(v_cache + (slot * G + g) * Dv + 8 * c);
+            }
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                Vt[(8 * c + 2 * e) * vst + j] = (bf16s)(w[e] & 0xffffu);
+                Vt[(8 * c + 2 * e + 1) * vst + j] = (bf16s)(w[e] >> 16);
+            }
+        }
+        __syncthreads();
+        if (ntok <= 0 || k0 > wave_last) continue;
+        // S^T tiles: keys k0 + 16*mt + 4*lg + r, token lc
+        f4_t sc[4];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            sc[mt] = f4_t{0.f, 0.f, 0.f, 0.f};
+            const bf16s* kr = Ks + (16 * mt + lc) * kst + 4 * lg;
+#pragma unroll
+            for (int ks = 0; ks < MAXD; ++ks)
+                if (16 * ks < D)
+                    sc[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                        *reinterpret_cast<const s4_t*>(kr + 16 * ks), qf[ks], sc[mt], 0, 0, 0);
+        }
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = k0 + 16 * mt + 4 * lg + r;
+                float v = sc[mt][r] * scale - slope * (float)(pos - key);
+                v = (key <= pos) ? v : -INFINITY;
+                sc[mt][r] = v;
+                mloc = fmaxf(mloc, v);
+            }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+        const float mnew = fmaxf(m, mloc);
+        const float corr = (m == -INFINITY) ? 0.0f : expf(m - mnew);
+        float lsum = 0.0f;
+        s4_t phi[4], plo[4];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float v = sc[mt][r];
+                const float p = (v == -INFINITY) ? 0.0f : expf(v - mnew);
+                lsum += p;
+                const bf16s hi = f32_to_bf16(p);
+                phi[mt][r] = (short)hi;
+                plo[mt][r] = (short)f32_to_bf16(p - bf16_to_f32(hi));
+            }
+        lsum += __shfl_xor(lsum, 16, WAVE);
+        lsum += __shfl_xor(lsum, 32, WAVE);
+        l = l * corr + lsum;
+        m = mnew;
+#pragma unroll
+        for (int dt = 0; dt < MAXDV; ++dt) {
+            if (16 * dt < Dv) {
+                o[dt] *= corr;
+                const bf16s* vr = Vt + (16 * dt + lc) * vst + 4 * lg;
+#pragma unroll
+                for (int mt = 0; mt < 4; ++mt) {
+                    const s4_t a = *reinterpret_cast<const s4_t*>(vr + 16 * mt);
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, phi[mt], o[dt], 0, 0, 0);
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, plo[mt], o[dt], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (lc >= ntok) return;
+    const int tok = lo + t0 + lc;
+    if (nsplit == 1) {
+        const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) / l;
+        bf16s* orow = out + ((int64_t)tok * H + h) * Dv + 4 * lg;
+#pragma unroll
+        for (int dt = 0; dt < MAXDV; ++dt)
+            if (16 * dt < Dv) {
+                uint2 w;
+                w.x = pack_bf16x2(o[dt][0] * gt, o[dt][1] * gt);
+                w.y = pack_bf16x2(o[dt][2] * gt, o[dt][3] * gt);
+                *reinterpret_cast<uint2*>(orow + 16 * dt) = w;
+            }
+    } else {
+        const int64_t pr = ((int64_t)tok * H + h) * nsplit + split;
+#pragma unroll
+        for (int dt = 0; dt < MAXDV; ++dt)
+            if (16 * dt < Dv)
+                *reinterpret_cast<f4_t*>(part_o + pr * Dv + 16 * dt + 4 * lg) = o[dt];
+        if (lg == 0) {
+            part_ml[pr * 2] = m;
+            part_ml[pr * 2 + 1] = l;
+        }
+    }
+}
+
 // merge key-split partials: one wave per (token, head)
 template <typename TC>
 __global__ __launch_bounds__(64) void attn_combine_kernel(
@@ -628,11 +823,26 @@ extern "C" int oa_attn_prepare(void* stream, const void* qkv, int64_t qs, const 
     return 0;
 }
 
-// Geometry the host must agree with: tile size, key-tile size, LDS bytes.
+// Which kernel serves a shape, and the geometry the host must agree with:
+// query tokens per tile (TQ), keys per staged tile (KT), K row stride, LDS
+// bytes. path 1 = matrix cores (bf16, sizes multiples of 16), 0 = VALU.
+static int attn_path(int H, int G, int D, int Dv, int dt) {
+    if (std::getenv("OPSAGENT_ATTN_VALU")) return 0;
+    return (dt == 0 && D % 16 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256) ? 1 : 0;
+}
+static int attn_hb(int R) { return R % 4 == 0 ? 4 : (R % 2 == 0 ? 2 : 1); }
+
 extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int* TQ, int* KT,
                                      int* kstride, int* lds_bytes) {
     if (G < 1 || H % G != 0 || Dv > 64 * ATT_MAXV) return -100;
     const int R = H / G;
+    if (attn_path(H, G, D, Dv, dt)) {
+        *TQ = 16 * (4 / attn_hb(R));
+        *KT = MF_KT;
+        *kstride = D + 4;
+        *lds_bytes = (MF_KT * (D + 4) + Dv * (MF_KT + 4)) * 2;
+        return 0;
+    }
     if (R > 4 * ATT_MAXR) return -102;
     int tq = std::max(1, (4 * ATT_MAXR) / R);
     const int esz = dt == 1 ? 4 : 2;
@@ -649,6 +859,23 @@ extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int* T
     return -103;
 }
 
+template <int MAXD, int MAXDV>
+static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void* q, const void* gate,
+                             int64_t gs, const void* k_cache, const void* v_cache, void* out,
+                             void* part_o, void* part_ml, const void* cu, const void* past,
+                             const void* block_table, int max_blocks, int block_size,
+                             const void* slopes, int B, int H, int G, int D, int Dv, int HB,
+                             float scale, int nsplit) {
+    if (lds_bytes > 48 * 1024)
+        (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    hipLaunchKernelGGL((attn_bias_mfma_kernel<MAXD, MAXDV>), grid, dim3(256), lds_bytes, s,
+                       (const bf16s*)q, (const bf16s*)gate, gs, (const bf16s*)k_cache,
+                       (const bf16s*)v_cache, (bf16s*)out, (float*)part_o, (float*)part_ml,
+                       (const int*)cu, (const int*)past, (const int*)block_table, max_blocks,
+                       block_size, (const float*)slopes, B, H, G, D, Dv, HB, scale, nsplit);
+}
+
 // ntiles = sum_b ceil(n_b / TQ) (host-computed). part_* may be null when nsplit == 1.
 extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate, int64_t gs,
                                   const void* k_cache, const void* v_cache, void* out,
@@ -662,18 +889,38 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
     if (rc) return rc;
     if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return -104;
     hipStream_t s = (hipStream_t)stream;
-    dim3 grid(ntiles, G, nsplit), blk(256);
+    if (attn_path(H, G, D, Dv, dt)) {
+        const int R = H / G, HB = attn_hb(R);
+        dim3 grid(ntiles, G * (R / HB), nsplit);
+#define MF(A, Bv) launch_attn_mfma<A, Bv>(s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out, part_o, \
+                                          part_ml, cu, past, block_table, max_blocks, block_size, slopes, \
+                                          B, H, G, D, Dv, HB, scale, nsplit)
+        const int a = D <= 64 ? 4 : (D <= 128 ? 8 : 16), bv = Dv <= 64 ? 4 : (Dv <= 128 ? 8 : 16);
+        if (a == 4 && bv == 4) MF(4, 4);
+        else if (a == 4 && bv == 8) MF(4, 8);
+        else if (a == 4) MF(4, 16);
+        else if (a == 8 && bv == 4) MF(8, 4);
+        else if (a == 8 && bv == 8) MF(8, 8);
+        else if (a == 8) MF(8, 16);
+        else if (bv == 4) MF(16, 4);
+        else if (bv == 8) MF(16, 8);
+        else MF(16, 16);
+#undef MF
+        HIP_CHECK_LAUNCH();
+    } else {
+        dim3 grid(ntiles, G, nsplit), blk(256);
 #define AT_ARGS(TC)                                                                      \
     (const TC*)q, (const TC*)gate, gs, (const TC*)k_cache, (const TC*)v_cache, (TC*)out,  \
         (float*)part_o, (float*)part_ml, (const int*)cu, (const int*)past,                \
         (const int*)block_table, max_blocks, block_size, (const float*)slopes, B, H, G, D, \
         Dv, TQ, KT, ks, scale, nsplit
-    if (dt == 1)
-        hipLaunchKernelGGL((attn_bias_paged_kernel<float>), grid, blk, lds_bytes, s, AT_ARGS(float));
-    else
-        hipLaunchKernelGGL((attn_bias_paged_kernel<bf16s>), grid, blk, lds_bytes, s, AT_ARGS(bf16s));
+        if (dt == 1)
+            hipLaunchKernelGGL((attn_bias_paged_kernel<float>), grid, blk, lds_bytes, s, AT_ARGS(float));
+        else
+            hipLaunchKernelGGL((attn_bias_paged_kernel<bf16s>), grid, blk, lds_bytes, s, AT_ARGS(bf16s));
 #undef AT_ARGS
-    HIP_CHECK_LAUNCH();
+        HIP_CHECK_LAUNCH();
+    }
     if (nsplit > 1) {
         if (dt == 1)
             hipLaunchKernelGGL((attn_combine_kernel<float>), dim3((unsigned)((int64_t)T * H)), dim3(64), 0, s,

@@ -1,0 +1,98 @@
+"""Prefill and decode throughput of a hybrid decoder beside the llama model
+of equal width, depth, head geometry and feed-forward size (random weights,
+random token ids). Used by `bench.py --mode layers`.
+
+For each size both engines get the same workload through the same public
+path (add_request + step): B prompts of P tokens are read, then D tokens are
+decoded greedily per request. Prefill tokens/s = B*P / time until every
+prompt is read; decode tokens/s = B*D / time of the decode steps.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import time
+from typing import Dict, List
+
+import torch
+
+from opsagent_amd.engine.config import ModelSpec, povazen_config_dict, povazen_spec_from_dict
+
+# (name, width, heads, kv_heads, head dim, ff, layers)
+SIZES = [
+    ("1b-class", 2048, 16, 4, 128, 8192, 4),
+    ("8b-class", 4096, 32, 8, 128, 14336, 4),
+]
+
+
+def specs_for(size) -> Dict[str, object]:
+    name, width, heads, kv, dim, ff, layers = size
+    llama = ModelSpec(
+        name=f"llama-{name}", vocab_size=32000, hidden_size=width, intermediate_size=ff,
+        num_layers=layers, num_heads=heads, num_kv_heads=kv, head_dim=dim, max_seq_len=8192,
+    )
+    pattern = ("da" * layers)[:layers]           # delta and attention layers alternate
+    hybrid = povazen_spec_from_dict(
+        povazen_config_dict(vocab=32000, width=width, pattern=pattern, heads=heads,
+                            kv_heads=kv, dim=dim, vdim=dim, ff=ff, delta_heads=heads),
+        name=f"povazen-{name}",
+    )
+    return {"llama": llama, "povazen": hybrid}
+
+
+def _run(spec, batch: int, prompt: int, decode: int, reps: int) -> Dict[str, float]:
+    from opsagent_amd.engine.engine import LLMEngine, SamplingParams
+
+    eng = LLMEngine({
+        "model": spec, "dtype": "bf16", "kv_block_size": 32,
+        "kv_num_blocks": max(64, 2 * batch * ((prompt + decode) // 32 + 2)),
+        "max_batch_size": max(batch, 1), "max_seq_len": 8192, "max_prefill_chunk": 8192,
+        "tokenizer_check": False, "spec_decode": False, "seed": 7,
+    })
+    gen = torch.Generator().manual_seed(0)
+    params = SamplingParams(max_new_tokens=decode, stop_on_eos=False)
+    pre_s: List[float] = []
+    dec_s: List[float] = []
+    for rep in range(reps + 1):                  # first repetition warms up
+        prompts = [torch.randint(300, 30000, (prompt,), generator=gen).tolist()
+                   for _ in range(batch)]
+        rids = [eng.add_request(p, params) for p in prompts]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while any(len(eng.requests[r].output_ids) == 0 for r in rids):
+            eng.step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        while not all(eng.requests[r].finished for r in rids):
+            eng.step()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for r in rids:
+            eng.requests.pop(r)
+        if rep:
+            pre_s.append(t1 - t0)
+            dec_s.append(t2 - t1)
+    pre, dec = min(pre_s), min(dec_s)
+    del eng
+    torch.cuda.empty_cache()
+    return {"prefill_tok_s": batch * prompt / pre, "decode_tok_s": batch * (decode - 1) / dec,
+            "prefill_ms": pre * 1e3, "decode_ms_per_step": dec * 1e3 / (decode - 1)}
+
+
+def run(sizes=None, prompt: int = 2048, decode: int = 64, batches=(1, 8), reps: int = 2,
+        models=("llama", "povazen")) -> List[dict]:
+    rows = []
+    for size in (sizes or SIZES):
+        specs = specs_for(size)
+        for b in batches:
+            row = {"size": size[0], "batch": b, "prompt": prompt, "decode": decode}
+            for m in models:
+                r = _run(specs[m], b, prompt, decode, reps)
+                row[m] = {k: round(v, 2) for k, v in r.items()}
+            if "llama" in row and "povazen" in row:
+                row["povazen_vs_llama"] = {
+                    "prefill": round(row["povazen"]["prefill_tok_s"] / row["llama"]["prefill_tok_s"], 3),
+                    "decode": round(row["povazen"]["decode_tok_s"] / row["llama"]["decode_tok_s"], 3),
+                }
+            rows.append(row)
+    return rows

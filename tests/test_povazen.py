@@ -45,7 +45,7 @@ def close(got, want, dtype, what=""):
     err = (got - want).pow(2).mean().sqrt() / (want.pow(2).mean().sqrt() + 1e-9)
     worst = (got - want).abs().max() / (want.abs().max() + 1e-9)
     if dtype == "fp32":
-        assert err < 2e-5 and worst < 2e-4, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
+        assert err < 5e-4 and worst < 2e-3, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
     else:
         assert err < 3e-2 and worst < 1.5e-1, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
 
@@ -195,22 +195,34 @@ def _single_layer(kind, dtype, device, seed=0, **kw):
     return cfg, rounded(W, dtype), eng
 
 
+# (heads, kv_heads, dim, vdim): ratios 1..4 and sizes that do and do not
+# divide by 16 (matrix-core and VALU kernels on the GPU)
+ATT_GEOMS = [(6, 2, 24, 40), (6, 2, 32, 48), (8, 2, 16, 80), (4, 2, 64, 16), (2, 2, 160, 32),
+             (3, 1, 144, 144)]
+
+
 @pytest.mark.parametrize("mode", MODES)
-def test_attention_mixer_alone(mode):
+@pytest.mark.parametrize("geom", ATT_GEOMS)
+def test_attention_mixer_alone(mode, geom):
     """The mixer module on a given input h, through the paged cache, in one
     portion and in uneven portions."""
     device, dtype = mode
     _skip_if_wrong_device(device)
-    cfg, W, eng = _single_layer("A", dtype, device)
+    hq, hk, dim, vdim = geom
+    cfg, W, eng = _single_layer("A", dtype, device, heads=hq, kv_heads=hk, dim=dim, vdim=vdim)
     mixer = eng.model.layers[0].mixer
     g = torch.Generator().manual_seed(5)
     T = 37
     h = torch.randn(T, cfg["width"], generator=g).to(tdtype(dtype))
     want = O.attention_mixer(h.double(), {k: v.double() for k, v in W.items()}, "l0.mix.",
                              cfg["layers"][0]["mixer"], cfg["norm"]["eps"])
-    for sizes in ([T], [5, 2, 9, 1, 1, 16, 3]):
+    T = 85
+    h = torch.randn(T, cfg["width"], generator=g).to(tdtype(dtype))
+    want = O.attention_mixer(h.double(), {k: v.double() for k, v in W.items()}, "l0.mix.",
+                             cfg["layers"][0]["mixer"], cfg["norm"]["eps"])
+    for sizes in ([T], [5, 2, 9, 1, 1, 16, 3, 40, 8]):
         outs, at = [], 0
-        blocks = [9, 2, 5, 11, 4]
+        blocks = [9, 2, 5, 11, 4, 30, 17, 1, 22, 6, 13]
         for n in sizes:
             sb, _ = one_seq_batch(n, at, eng.device, blocks=blocks)
             outs.append(mixer(h[at:at + n].to(eng.device), sb, eng.kv.layers[0], eng.state_pool.tensors[0]))
@@ -261,14 +273,15 @@ def test_delta_decay_and_beta_extremes(mode):
 
 
 @pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("vdim", [12, 16])
 @pytest.mark.parametrize("hot", [0, 1, 7, 8, 9, 31, 32, 63, 64, 100])
-def test_far_key_stands_out(mode, hot):
+def test_far_key_stands_out(mode, hot, vdim):
     """One key, far back or at a page border, is made to dominate the last
     query's softmax; a lost page, an off-by-one in the block table or in the
     distance penalty moves the output visibly. Prompt and decoded query."""
     device, dtype = mode
     _skip_if_wrong_device(device)
-    cfg, W, eng = _single_layer("A", dtype, device, heads=2, kv_heads=2, dim=16, vdim=12, scale=6.0)
+    cfg, W, eng = _single_layer("A", dtype, device, heads=2, kv_heads=2, dim=16, vdim=vdim, scale=6.0)
     # q and k share weights and have no bias: equal inputs give parallel q, k
     W["l0.mix.k"] = W["l0.mix.q"].clone()
     W["l0.mix.k.norm"] = W["l0.mix.q.norm"].clone()
@@ -297,9 +310,14 @@ def test_far_key_stands_out(mode, hot):
 # whole model through the engine
 
 
-@pytest.fixture(scope="module")
-def model_case():
-    cfg = make_cfg()
+@pytest.fixture(scope="module", params=["odd", "x16"])
+def model_case(request):
+    """'odd': sizes that divide by nothing much; 'x16': key/value sizes that
+    the matrix-core attention kernel takes."""
+    if request.param == "odd":
+        cfg = make_cfg()
+    else:
+        cfg = make_cfg(dim=32, vdim=48, heads=8, kv_heads=2, d_dim=32, d_vdim=16)
     W = other_ranks(cfg, O.random_weights(cfg, seed=1))
     return cfg, W
 
