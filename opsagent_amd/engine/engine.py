@@ -663,53 +663,58 @@ class LLMEngine:
 
     def _mixed_decode_graphed(self, ids: List[int], chunks) -> torch.Tensor:
         """Decode-only step of a hybrid model through a hipGraph captured per
-        batch bucket: static SeqBatch tensors are refilled, padding rows
-        repeat row 0 (same token, same slots: an idempotent rewrite is NOT
-        safe for recurrent state, so padded rows get count 0 instead)."""
+        batch bucket: static SeqBatch tensors are refilled; padding rows get
+        a count of 0 (repeating row 0, as the llama path does, would apply
+        its recurrent update twice)."""
         from opsagent_amd.ops.mixer_ops import SeqBatch
 
         B = len(chunks)
         bucket = self._bucket(B)
         ent = self._graphs.get(bucket)
+        mb = self.max_blocks_per_seq
+        # flat int32 layout: cu | past | slots | seq_of | slot_map | block table
+        o1, o2, o3, o4, o5 = (bucket + 1, 2 * bucket + 1, 3 * bucket + 1,
+                              4 * bucket + 1, 5 * bucket + 1)
         if ent is None:
             dev = self.device
-            i32 = torch.int32
+            flat = torch.zeros(o5 + bucket * mb, dtype=torch.int32, device=dev)
             sb = SeqBatch(
                 cu=list(range(bucket + 1)), past=[0] * bucket, slots=[0] * bucket,
-                cu_t=torch.zeros(bucket + 1, dtype=i32, device=dev),
-                past_t=torch.zeros(bucket, dtype=i32, device=dev),
-                slots_t=torch.zeros(bucket, dtype=i32, device=dev),
-                seq_of_t=torch.arange(bucket, dtype=i32, device=dev),
-                slot_mapping=torch.zeros(bucket, dtype=i32, device=dev),
-                block_table=torch.zeros(bucket, self.max_blocks_per_seq, dtype=i32, device=dev),
-                max_chunk=1,
-                max_total=self.max_blocks_per_seq * self.block_size,
+                cu_t=flat[:o1], past_t=flat[o1:o2], slots_t=flat[o2:o3],
+                seq_of_t=flat[o3:o4], slot_mapping=flat[o4:o5],
+                block_table=flat[o5:].view(bucket, mb),
+                max_chunk=1, max_total=mb * self.block_size,
             )
-            ids_t = torch.zeros(bucket, dtype=torch.int64, device=dev)
-            ent = {"sb": sb, "ids": ids_t, "graph": None, "out": None}
+            ent = {
+                "sb": sb, "flat": flat, "graph": None, "out": None,
+                "ids": torch.zeros(bucket, dtype=torch.int64, device=dev),
+                "h_flat": torch.zeros(o5 + bucket * mb, dtype=torch.int32, pin_memory=True),
+                "h_ids": torch.zeros(bucket, dtype=torch.int64, pin_memory=True),
+            }
             self._graphs[bucket] = ent
         sb, ids_t = ent["sb"], ent["ids"]
-        # host staging -> static device tensors. Padding rows: zero tokens
-        # (cu stays flat), so no kernel touches any state for them.
-        cu = [min(i, B) for i in range(bucket + 1)]
-        past = [c[0] for c in chunks] + [0] * (bucket - B)
-        slots = [c[2] for c in chunks] + [0] * (bucket - B)
+        # persistent pinned staging -> two copies per step. Padding rows hold
+        # zero tokens (cu stays flat), so no kernel touches any state for
+        # them. sb's HOST lists stay at the bucket's upper bound (one token
+        # per row): they only size launches; kernels read the device copies.
+        hf = ent["h_flat"].numpy()
         bs = self.block_size
+        hf[:o1] = [min(i, B) for i in range(bucket + 1)]
+        hf[o1:o5] = 0
+        hf[o1 : o1 + B] = [c[0] for c in chunks]
+        hf[o2 : o2 + B] = [c[2] for c in chunks]
+        hf[o3 : o3 + B] = range(B)
         slot_map = [c[3][c[0] // bs] * bs + c[0] % bs for c in chunks]
-        slot_map += [slot_map[0]] * (bucket - B)
-        seq_of = list(range(B)) + [0] * (bucket - B)
-        bt = torch.zeros(bucket, self.max_blocks_per_seq, dtype=torch.int32)
+        hf[o4:o5] = slot_map[0]
+        hf[o4 : o4 + B] = slot_map
         for b, c in enumerate(chunks):
-            bt[b, : len(c[3])] = torch.tensor(c[3], dtype=torch.int32)
-        # sb's HOST lists stay at the bucket's upper bound (one token per
-        # row): they only size launches; the kernels read the device copies
-        sb.cu_t.copy_(torch.tensor(cu, dtype=torch.int32))
-        sb.past_t.copy_(torch.tensor(past, dtype=torch.int32))
-        sb.slots_t.copy_(torch.tensor(slots, dtype=torch.int32))
-        sb.seq_of_t.copy_(torch.tensor(seq_of, dtype=torch.int32))
-        sb.slot_mapping.copy_(torch.tensor(slot_map, dtype=torch.int32))
-        sb.block_table.copy_(bt)
-        ids_t.copy_(torch.tensor(ids + [ids[0]] * (bucket - B), dtype=torch.int64))
+            hf[o5 + b * mb : o5 + b * mb + len(c[3])] = c[3]
+        hi = ent["h_ids"].numpy()
+        hi[:] = ids[0]
+        hi[:B] = ids
+        # blocking copies: the staging buffers are rewritten next step
+        ent["flat"].copy_(ent["h_flat"])
+        ids_t.copy_(ent["h_ids"])
         fb = ForwardBatch(kind="mixed", input_ids=ids_t, positions=None,
                           slot_mapping=sb.slot_mapping, seq_batch=sb)
         if ent["graph"] is None:

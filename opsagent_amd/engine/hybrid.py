@@ -144,10 +144,10 @@ class ChannelDeltaMixer(nn.Module):
         g1 = proj[:, o0 + H + self.ra :]
         a = ops.linear(a1, self.a2_w)                         # [T, H*D]
         gate = ops.linear(g1, self.g2_w)                      # [T, H*Dv]
-        o = mx.channel_delta_rule(
+        y = mx.channel_delta_rule(
             qkv[:, : G * D], qkv[:, G * D : 2 * G * D], qkv[:, 2 * G * D :],
-            b_logits, a, self.dt_bias, self.a_log, state["S"], sb, H, G, D, Dv)
-        y = mx.gated_head_rms_norm(o, self.norm_w, gate, self.eps)
+            b_logits, a, self.dt_bias, self.a_log, self.norm_w, gate, state["S"], sb,
+            H, G, D, Dv, self.eps)
         return ops.linear(y, self.o_w)
 
 

@@ -95,6 +95,48 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
     }
 }
 
+// Convolution and carry in ONE launch for steps whose portions are a few
+// tokens (decoding): one thread per (sequence, channel) walks its tokens in
+// order and then rewrites its own column of the carried inputs, so no other
+// thread reads what it overwrites.
+template <typename TI, typename TW, typename TO>
+__global__ __launch_bounds__(256) void causal_conv_small_kernel(
+    const TI* __restrict__ x, int64_t xs, const TW* __restrict__ w,
+    float* __restrict__ state, TO* __restrict__ out, int64_t os,
+    const int* __restrict__ cu, const int* __restrict__ past,
+    const int* __restrict__ slots, int B, int C, int taps, int add_input,
+    int act_silu) {
+    const int64_t total = (int64_t)B * C;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int b = (int)(idx / C), c = (int)(idx % C);
+        const int lo = cu[b], n = cu[b + 1] - lo;
+        if (n <= 0) continue;
+        const int p = past[b];
+        float* st = state + (int64_t)slots[b] * (taps - 1) * C;
+        for (int i = 0; i < n; ++i) {
+            float acc = 0.0f;
+            for (int j = 0; j < taps; ++j) {
+                const int s = i + j - (taps - 1);
+                if (p + s < 0) continue;
+                const float xv = (s >= 0) ? ldf(x, (int64_t)(lo + s) * xs + c)
+                                          : st[(int64_t)(taps - 1 + s) * C + c];
+                acc += ldf(w, (int64_t)c * taps + j) * xv;
+            }
+            if (add_input) acc += ldf(x, (int64_t)(lo + i) * xs + c);
+            if (act_silu) acc = acc * sigmoidf_(acc);
+            stf(out, (int64_t)(lo + i) * os + c, acc);
+        }
+        for (int i = 0; i < taps - 1; ++i) {
+            const int local = n - (taps - 1) + i;
+            float v;
+            if (local >= 0) v = ldf(x, (int64_t)(lo + local) * xs + c);
+            else v = (p + local < 0) ? 0.0f : st[(int64_t)(i + n) * C + c];
+            st[(int64_t)i * C + c] = v;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // RMS norm in `groups` consecutive parts, times w; one block per token, one
 // wave per part. residual (float32, may be null) is updated in place:
@@ -560,71 +602,49 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Delta-rule preparation, one block per token (all float32 outputs):
-//   qn = q / sqrt(sum q^2 + 1e-6) * D^-1/2,  kn = k / sqrt(sum k^2 + 1e-6)
-//   decay[h, d] = exp(-exp(A_log[h]) * softplus(a[h, d] + dt_bias[h, d]))
-//   beta[h] = sigmoid(b[h])
-template <typename TC>
-__global__ __launch_bounds__(256) void delta_prepare_kernel(
-    const TC* __restrict__ q, int64_t qs, const TC* __restrict__ k, int64_t ks,
-    const TC* __restrict__ bl, int64_t bs, const TC* __restrict__ a, int64_t as,
-    const TC* __restrict__ dt_bias, const TC* __restrict__ a_log,
-    float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ decay,
-    float* __restrict__ beta, int H, int G, int D) {
-    const int t = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const float qscale = 1.0f / sqrtf((float)D);
-    for (int u = wave; u < 2 * G; u += nw) {
-        const int g = u >> 1;
-        const bool is_q = (u & 1) == 0;
-        const TC* src = is_q ? q + (int64_t)t * qs + g * D : k + (int64_t)t * ks + g * D;
-        float* dst = (is_q ? qn : kn) + ((int64_t)t * G + g) * D;
-        float ss = 0.0f;
-        for (int i = lane; i < D; i += 64) {
-            float v = ldf(src, i);
-            ss += v * v;
-        }
-        ss = wave_reduce_sum(ss);
-        const float r = (1.0f / sqrtf(ss + 1e-6f)) * (is_q ? qscale : 1.0f);
-        for (int i = lane; i < D; i += 64) dst[i] = ldf(src, i) * r;
-    }
-    for (int i = threadIdx.x; i < H * D; i += blockDim.x) {
-        const int h = i / D;
-        const float z = ldf(a, (int64_t)t * as + i) + ldf(dt_bias, i);
-        decay[(int64_t)t * H * D + i] = expf(-expf(ldf(a_log, h)) * softplusf_(z));
-    }
-    for (int h = threadIdx.x; h < H; h += blockDim.x)
-        beta[(int64_t)t * H + h] = sigmoidf_(ldf(bl, (int64_t)t * bs + h));
-}
-
-// The recurrence. grid = (sequences, heads, value-column groups of 16), one
-// wave per block. Lane = (column, row group): 16 columns x 4 row groups,
-// each lane holds RPL consecutive key rows of its column of S in registers.
-// Per token:  S <- decay * S;  u = beta * (v - S^T k);  S <- S + k u^T;
-// o = S^T q   (the read-out sees the token's own write).
-// q, k, decay of DR_TC tokens at a time are staged in LDS (rows past D are
-// staged as zero so the inner loops need no bounds).
-#define DR_TC 16
+// Gated delta rule with one decay per head and key channel, fused from the
+// convolved q/k/v to the gated, normed read-out. grid = (sequences, heads);
+// a block has one wave per 16 value columns. Lane = (column, row group): 16
+// columns x 4 row groups, each lane holds RPL consecutive key rows of its
+// column of S in registers (S lives in float32 in the state slot between
+// steps; a sequence that starts at position 0 starts from zero whatever
+// the slot holds).
+// Per chunk of TCK tokens the block
+//   1. stages q, k (raw), decay = exp(-exp(A_log) softplus(a + dt_bias)),
+//      v and beta = sigmoid(b) in LDS as float32 (rows past D as zero),
+//   2. makes q and k unit vectors (q also times D^-1/2), a wave per token,
+//   3. runs the recurrence, every wave on its own columns:
+//        S <- decay * S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//   4. RMS-norms o over the head's value columns, times w, times
+//      sigmoid(gate), a wave per token, and stores it.
 template <int RPL, typename TC>
-__global__ __launch_bounds__(64) void delta_recurrent_kernel(
-    const float* __restrict__ qn, const float* __restrict__ kn,
-    const float* __restrict__ decay, const float* __restrict__ beta,
-    const TC* __restrict__ v, int64_t vs, float* __restrict__ state,
-    float* __restrict__ out, const int* __restrict__ cu,
-    const int* __restrict__ past, const int* __restrict__ slots, int H, int G,
-    int D, int Dv) {
+__global__ void delta_fused_kernel(
+    const TC* __restrict__ q, int64_t qs, const TC* __restrict__ k, int64_t ks,
+    const TC* __restrict__ v, int64_t vs, const TC* __restrict__ bl, int64_t bs,
+    const TC* __restrict__ a, int64_t as, const TC* __restrict__ dt_bias,
+    const TC* __restrict__ a_log, const TC* __restrict__ norm_w,
+    const TC* __restrict__ gate, int64_t gs, float* __restrict__ state,
+    TC* __restrict__ out, const int* __restrict__ cu, const int* __restrict__ past,
+    const int* __restrict__ slots, int H, int G, int D, int Dv, int TCK, float eps) {
     constexpr int DP = RPL * 4;  // padded key size
-    __shared__ float sq[DR_TC][DP];
-    __shared__ float sk[DR_TC][DP];
-    __shared__ float sg[DR_TC][DP];
+    extern __shared__ float lds[];
+    float* sq = lds;
+    float* sk = sq + TCK * DP;
+    float* sg = sk + TCK * DP;
+    float* sv = sg + TCK * DP;
+    float* so = sv + TCK * Dv;
+    float* sb = so + TCK * Dv;
     const int b = blockIdx.x, h = blockIdx.y;
-    const int lane = threadIdx.x;
-    const int col = blockIdx.z * 16 + (lane & 15), rg = lane >> 4;
+    const int tid = threadIdx.x, nth = blockDim.x;
+    const int lane = tid & 63, wave = tid >> 6, nw = nth >> 6;
+    const int col = wave * 16 + (lane & 15), rg = lane >> 4;
     const bool col_ok = col < Dv;
     const int lo = cu[b], n = cu[b + 1] - lo;
     if (n <= 0) return;
     const int kvh = h / (H / G);
     float* st = state + (((int64_t)slots[b] * H + h) * D) * Dv;
+    const float A = expf(ldf(a_log, h));
+    const float qscale = 1.0f / sqrtf((float)D);
     float S[RPL];
     const bool fresh = past[b] == 0;
 #pragma unroll
@@ -632,26 +652,52 @@ __global__ __launch_bounds__(64) void delta_recurrent_kernel(
         const int r = rg * RPL + i;
         S[i] = (!fresh && col_ok && r < D) ? st[(int64_t)r * Dv + col] : 0.0f;
     }
-    for (int c0 = 0; c0 < n; c0 += DR_TC) {
-        const int nc = min(DR_TC, n - c0);
-        __builtin_amdgcn_wave_barrier();
-        for (int i = lane; i < nc * DP; i += 64) {
+    for (int c0 = 0; c0 < n; c0 += TCK) {
+        const int nc = min(TCK, n - c0);
+        const int tb = lo + c0;
+        for (int i = tid; i < nc * DP; i += nth) {
             const int tt = i / DP, r = i % DP;
-            const int t = lo + c0 + tt;
-            const bool ok = r < D;
-            sq[tt][r] = ok ? qn[((int64_t)t * G + kvh) * D + r] : 0.0f;
-            sk[tt][r] = ok ? kn[((int64_t)t * G + kvh) * D + r] : 0.0f;
-            sg[tt][r] = ok ? decay[((int64_t)t * H + h) * D + r] : 0.0f;
+            const int64_t t = tb + tt;
+            float qv = 0.0f, kv = 0.0f, gv = 0.0f;
+            if (r < D) {
+                qv = ldf(q, t * qs + kvh * D + r);
+                kv = ldf(k, t * ks + kvh * D + r);
+                const float z = ldf(a, t * as + h * D + r) + ldf(dt_bias, h * D + r);
+                gv = expf(-A * softplusf_(z));
+            }
+            sq[i] = qv;
+            sk[i] = kv;
+            sg[i] = gv;
         }
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_wave_barrier();
+        for (int i = tid; i < nc * Dv; i += nth) {
+            const int tt = i / Dv, c = i % Dv;
+            sv[i] = ldf(v, (int64_t)(tb + tt) * vs + h * Dv + c);
+        }
+        for (int tt = tid; tt < nc; tt += nth)
+            sb[tt] = sigmoidf_(ldf(bl, (int64_t)(tb + tt) * bs + h));
+        __syncthreads();
+        for (int tt = wave; tt < nc; tt += nw) {
+            float ssq = 0.0f, ssk = 0.0f;
+            for (int i = lane; i < DP; i += 64) {
+                const float x = sq[tt * DP + i], y = sk[tt * DP + i];
+                ssq += x * x;
+                ssk += y * y;
+            }
+            ssq = wave_reduce_sum(ssq);
+            ssk = wave_reduce_sum(ssk);
+            const float rq = qscale / sqrtf(ssq + 1e-6f), rk = 1.0f / sqrtf(ssk + 1e-6f);
+            for (int i = lane; i < DP; i += 64) {
+                sq[tt * DP + i] *= rq;
+                sk[tt * DP + i] *= rk;
+            }
+        }
+        __syncthreads();
         for (int tt = 0; tt < nc; ++tt) {
-            const int t = lo + c0 + tt;
-            const float bt = beta[(int64_t)t * H + h];
-            const float vv = col_ok ? ldf(v, (int64_t)t * vs + (int64_t)h * Dv + col) : 0.0f;
-            const float* kq = &sk[tt][rg * RPL];
-            const float* gq = &sg[tt][rg * RPL];
-            const float* qq = &sq[tt][rg * RPL];
+            const float bt = sb[tt];
+            const float vv = col_ok ? sv[tt * Dv + col] : 0.0f;
+            const float* kq = sk + tt * DP + rg * RPL;
+            const float* gq = sg + tt * DP + rg * RPL;
+            const float* qq = sq + tt * DP + rg * RPL;
             float dot = 0.0f;
 #pragma unroll
             for (int i = 0; i < RPL; ++i) {
@@ -669,35 +715,27 @@ __global__ __launch_bounds__(64) void delta_recurrent_kernel(
             }
             o += __shfl_xor(o, 16, WAVE);
             o += __shfl_xor(o, 32, WAVE);
-            if (rg == 0 && col_ok) out[((int64_t)t * H + h) * Dv + col] = o;
+            if (rg == 0 && col_ok) so[tt * Dv + col] = o;
         }
+        __syncthreads();
+        for (int tt = wave; tt < nc; tt += nw) {
+            float ss = 0.0f;
+            for (int c = lane; c < Dv; c += 64) ss += so[tt * Dv + c] * so[tt * Dv + c];
+            ss = wave_reduce_sum(ss);
+            const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
+            const int64_t t = tb + tt;
+            for (int c = lane; c < Dv; c += 64) {
+                const float gt = sigmoidf_(ldf(gate, t * gs + h * Dv + c));
+                stf(out, (t * H + h) * Dv + c, so[tt * Dv + c] * r * ldf(norm_w, c) * gt);
+            }
+        }
+        // the next chunk's staging does not touch `so`, and its recurrence
+        // (which does) comes two barriers later
     }
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
         const int r = rg * RPL + i;
         if (col_ok && r < D) st[(int64_t)r * Dv + col] = S[i];
-    }
-}
-
-// per-head RMS norm of the read-out, times w[Dv], times sigmoid(gate):
-// one block per token, one wave per head
-template <typename TC>
-__global__ __launch_bounds__(256) void gated_head_norm_kernel(
-    const float* __restrict__ o, const TC* __restrict__ w,
-    const TC* __restrict__ gate, int64_t gs, TC* __restrict__ out, int H, int Dv,
-    float eps) {
-    const int t = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    for (int h = wave; h < H; h += nw) {
-        const float* src = o + ((int64_t)t * H + h) * Dv;
-        float ss = 0.0f;
-        for (int i = lane; i < Dv; i += 64) ss += src[i] * src[i];
-        ss = wave_reduce_sum(ss);
-        const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
-        for (int i = lane; i < Dv; i += 64) {
-            const float gt = sigmoidf_(ldf(gate, (int64_t)t * gs + h * Dv + i));
-            stf(out, ((int64_t)t * H + h) * Dv + i, src[i] * r * ldf(w, i) * gt);
-        }
     }
 }
 
@@ -752,11 +790,27 @@ extern "C" int oa_causal_conv_seq(void* stream, const void* x, int64_t xs, int x
                                   const void* w, void* state, void* out, int64_t os,
                                   const void* seq_of, const void* cu, const void* past,
                                   const void* slots, int T, int B, int C, int taps,
-                                  int add_input, int act_silu, int dt) {
+                                  int add_input, int act_silu, int dt, int max_chunk) {
     if (T <= 0) return 0;
     if (taps < 1) return -100;
     hipStream_t s = (hipStream_t)stream;
     dim3 g1(grid_for((int64_t)T * C)), g2(grid_for((int64_t)B * C)), blk(256);
+    if (max_chunk >= 1 && max_chunk <= 4) {
+#define CS_ARGS(TI, TW)                                                                      \
+    (const TI*)x, xs, (const TW*)w, (float*)state, (TW*)out, os, (const int*)cu,             \
+        (const int*)past, (const int*)slots, B, C, taps, add_input, act_silu
+        if (x_dt == 1 && dt == 1)
+            hipLaunchKernelGGL((causal_conv_small_kernel<float, float, float>), g2, blk, 0, s, CS_ARGS(float, float));
+        else if (x_dt == 1 && dt == 0)
+            hipLaunchKernelGGL((causal_conv_small_kernel<float, bf16s, bf16s>), g2, blk, 0, s, CS_ARGS(float, bf16s));
+        else if (x_dt == 0 && dt == 0)
+            hipLaunchKernelGGL((causal_conv_small_kernel<bf16s, bf16s, bf16s>), g2, blk, 0, s, CS_ARGS(bf16s, bf16s));
+        else
+            return -101;
+#undef CS_ARGS
+        HIP_CHECK_LAUNCH();
+        return 0;
+    }
 #define CONV_ARGS(TI, TW)                                                          \
     (const TI*)x, xs, (const TW*)w, (const float*)state, (TW*)out, os,             \
         (const int*)seq_of, (const int*)cu, (const int*)past, (const int*)slots, T, \
@@ -935,54 +989,48 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
     return 0;
 }
 
-extern "C" int oa_delta_prepare(void* stream, const void* q, int64_t qs, const void* k, int64_t ks,
-                                const void* bl, int64_t bs, const void* a, int64_t as,
-                                const void* dt_bias, const void* a_log, void* qn, void* kn,
-                                void* decay, void* beta, int T, int H, int G, int D, int dt) {
-    if (T <= 0) return 0;
-    hipStream_t s = (hipStream_t)stream;
-    if (dt == 1)
-        hipLaunchKernelGGL((delta_prepare_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)q, qs,
-                           (const float*)k, ks, (const float*)bl, bs, (const float*)a, as,
-                           (const float*)dt_bias, (const float*)a_log, (float*)qn, (float*)kn,
-                           (float*)decay, (float*)beta, H, G, D);
-    else
-        hipLaunchKernelGGL((delta_prepare_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const bf16s*)q, qs,
-                           (const bf16s*)k, ks, (const bf16s*)bl, bs, (const bf16s*)a, as,
-                           (const bf16s*)dt_bias, (const bf16s*)a_log, (float*)qn, (float*)kn,
-                           (float*)decay, (float*)beta, H, G, D);
-    HIP_CHECK_LAUNCH();
-    return 0;
-}
-
 template <int RPL>
-static int launch_delta(hipStream_t s, const void* qn, const void* kn, const void* decay,
-                        const void* beta, const void* v, int64_t vs, void* state, void* out,
-                        const void* cu, const void* past, const void* slots, int B, int H,
-                        int G, int D, int Dv, int dt) {
-    dim3 grid(B, H, CEIL_DIV(Dv, 16)), blk(64);
+static int launch_delta(hipStream_t s, const void* q, int64_t qs, const void* k, int64_t ks,
+                        const void* v, int64_t vs, const void* bl, int64_t bs, const void* a,
+                        int64_t as, const void* dt_bias, const void* a_log, const void* norm_w,
+                        const void* gate, int64_t gs, void* state, void* out, const void* cu,
+                        const void* past, const void* slots, int B, int H, int G, int D, int Dv,
+                        float eps, int dt) {
+    const int nw = CEIL_DIV(Dv, 16);
+    if (nw > 16) return -106;
+    int tck = 16;
+    auto bytes = [&](int t) { return (size_t)(3 * t * RPL * 4 + 2 * t * Dv + t) * 4; };
+    while (tck > 2 && bytes(tck) > 60 * 1024) tck >>= 1;
+    dim3 grid(B, H), blk(64 * nw);
+#define DARGS(TC)                                                                              \
+    (const TC*)q, qs, (const TC*)k, ks, (const TC*)v, vs, (const TC*)bl, bs, (const TC*)a, as,  \
+        (const TC*)dt_bias, (const TC*)a_log, (const TC*)norm_w, (const TC*)gate, gs,           \
+        (float*)state, (TC*)out, (const int*)cu, (const int*)past, (const int*)slots, H, G, D,  \
+        Dv, tck, eps
     if (dt == 1)
-        hipLaunchKernelGGL((delta_recurrent_kernel<RPL, float>), grid, blk, 0, s, (const float*)qn,
-                           (const float*)kn, (const float*)decay, (const float*)beta, (const float*)v,
-                           vs, (float*)state, (float*)out, (const int*)cu, (const int*)past,
-                           (const int*)slots, H, G, D, Dv);
+        hipLaunchKernelGGL((delta_fused_kernel<RPL, float>), grid, blk, bytes(tck), s, DARGS(float));
     else
-        hipLaunchKernelGGL((delta_recurrent_kernel<RPL, bf16s>), grid, blk, 0, s, (const float*)qn,
-                           (const float*)kn, (const float*)decay, (const float*)beta, (const bf16s*)v,
-                           vs, (float*)state, (float*)out, (const int*)cu, (const int*)past,
-                           (const int*)slots, H, G, D, Dv);
+        hipLaunchKernelGGL((delta_fused_kernel<RPL, bf16s>), grid, blk, bytes(tck), s, DARGS(bf16s));
+#undef DARGS
     HIP_CHECK_LAUNCH();
     return 0;
 }
 
-extern "C" int oa_delta_recurrent(void* stream, const void* qn, const void* kn, const void* decay,
-                                  const void* beta, const void* v, int64_t vs, void* state,
-                                  void* out, const void* cu, const void* past, const void* slots,
-                                  int T, int B, int H, int G, int D, int Dv, int dt) {
+// q, k [T, G*D], v [T, H*Dv], bl [T, H], a [T, H*D], gate [T, H*Dv]: rows with
+// the given strides; out [T, H*Dv] contiguous.
+extern "C" int oa_delta_rule_fused(void* stream, const void* q, int64_t qs, const void* k,
+                                   int64_t ks, const void* v, int64_t vs, const void* bl,
+                                   int64_t bs, const void* a, int64_t as, const void* dt_bias,
+                                   const void* a_log, const void* norm_w, const void* gate,
+                                   int64_t gs, void* state, void* out, const void* cu,
+                                   const void* past, const void* slots, int T, int B, int H, int G,
+                                   int D, int Dv, float eps, int dt) {
     if (T <= 0 || B <= 0) return 0;
     if (G < 1 || H % G != 0) return -100;
     hipStream_t s = (hipStream_t)stream;
-#define DL(R) launch_delta<R>(s, qn, kn, decay, beta, v, vs, state, out, cu, past, slots, B, H, G, D, Dv, dt)
+#define DL(R)                                                                                     \
+    launch_delta<R>(s, q, qs, k, ks, v, vs, bl, bs, a, as, dt_bias, a_log, norm_w, gate, gs, state, \
+                    out, cu, past, slots, B, H, G, D, Dv, eps, dt)
     if (D <= 32) return DL(8);
     if (D <= 64) return DL(16);
     if (D <= 96) return DL(24);
@@ -991,20 +1039,6 @@ extern "C" int oa_delta_recurrent(void* stream, const void* qn, const void* kn, 
     if (D <= 256) return DL(64);
 #undef DL
     return -105;
-}
-
-extern "C" int oa_gated_head_norm(void* stream, const void* o, const void* w, const void* gate,
-                                  int64_t gs, void* out, int T, int H, int Dv, float eps, int dt) {
-    if (T <= 0) return 0;
-    hipStream_t s = (hipStream_t)stream;
-    if (dt == 1)
-        hipLaunchKernelGGL((gated_head_norm_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)o,
-                           (const float*)w, (const float*)gate, gs, (float*)out, H, Dv, eps);
-    else
-        hipLaunchKernelGGL((gated_head_norm_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const float*)o,
-                           (const bf16s*)w, (const bf16s*)gate, gs, (bf16s*)out, H, Dv, eps);
-    HIP_CHECK_LAUNCH();
-    return 0;
 }
 
 extern "C" int oa_softcap(void* stream, const void* x, void* out, int64_t n, float cap, int dt) {

@@ -118,16 +118,14 @@ def _declare_mixers(lib: ctypes.CDLL) -> None:
     f = ctypes.c_float
     ip = ctypes.POINTER(ctypes.c_int)
     sigs = {
-        "oa_causal_conv_seq": [p, p, i64, i, p, p, p, i64, p, p, p, p, i, i, i, i, i, i, i],
+        "oa_causal_conv_seq": [p, p, i64, i, p, p, p, i64, p, p, p, p, i, i, i, i, i, i, i, i],
         "oa_group_rmsnorm": [p, p, i64, i, p, p, p, i, i, i, f, i],
         "oa_attn_prepare": [p, p, i64, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i],
         "oa_attn_bias_geometry": [i, i, i, i, i, ip, ip, ip, ip],
         "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p,
                                i, i, i, i, i, i, i, f, i, i],
-        "oa_delta_prepare": [p, p, i64, p, i64, p, i64, p, i64, p, p, p, p, p, p,
-                             i, i, i, i, i],
-        "oa_delta_recurrent": [p, p, p, p, p, p, i64, p, p, p, p, p, i, i, i, i, i, i, i],
-        "oa_gated_head_norm": [p, p, p, p, i64, p, i, i, i, f, i],
+        "oa_delta_rule_fused": [p, p, i64, p, i64, p, i64, p, i64, p, i64, p, p, p, p, i64,
+                                p, p, p, p, p, i, i, i, i, i, i, f, i],
         "oa_softcap": [p, p, p, i64, f, i],
         "oa_silu_mul_rows": [p, p, p, i64, i, i],
         "oa_embed_rows": [p, p, p, p, i, i, i],

@@ -50,10 +50,9 @@ class SeqBatch:
     def build(chunks: List[Tuple[int, int, int, List[int]]], block_size: int,
               device, max_blocks: Optional[int] = None) -> "SeqBatch":
         """chunks: per sequence (past_len, count, state_slot, block ids)."""
-        cu, past, slots, seq_of, slot_map = [0], [], [], [], []
+        cu, past, slots, seq_of, slot_map, bt = [0], [], [], [], [], []
         nb = max((len(c[3]) for c in chunks), default=1)
         max_blocks = max(max_blocks or 0, nb, 1)
-        bt = torch.zeros(len(chunks), max_blocks, dtype=torch.int32)
         for b, (p, n, slot, blocks) in enumerate(chunks):
             cu.append(cu[-1] + n)
             past.append(p)
@@ -61,16 +60,17 @@ class SeqBatch:
             seq_of.extend([b] * n)
             for pos in range(p, p + n):
                 slot_map.append(blocks[pos // block_size] * block_size + pos % block_size)
-            if blocks:
-                bt[b, : len(blocks)] = torch.tensor(blocks, dtype=torch.int32)
-
-        def dev(v):
-            return torch.tensor(v, dtype=torch.int32).to(device)
-
+            bt.extend(blocks)
+            bt.extend([0] * (max_blocks - len(blocks)))
+        # one host->device copy; the tensors are views of it
+        B, T = len(chunks), cu[-1]
+        flat = torch.tensor(cu + past + slots + seq_of + slot_map + bt,
+                            dtype=torch.int32).to(device)
+        o1, o2, o3, o4, o5 = B + 1, 2 * B + 1, 3 * B + 1, 3 * B + 1 + T, 3 * B + 1 + 2 * T
         return SeqBatch(
-            cu=cu, past=past, slots=slots, cu_t=dev(cu), past_t=dev(past),
-            slots_t=dev(slots), seq_of_t=dev(seq_of), slot_mapping=dev(slot_map),
-            block_table=bt.to(device),
+            cu=cu, past=past, slots=slots, cu_t=flat[:o1], past_t=flat[o1:o2],
+            slots_t=flat[o2:o3], seq_of_t=flat[o3:o4], slot_mapping=flat[o4:o5],
+            block_table=flat[o5:].view(B, max_blocks),
             max_chunk=max((c[1] for c in chunks), default=0),
             max_total=max((c[0] + c[1] for c in chunks), default=0),
         )
@@ -127,7 +127,7 @@ def causal_conv_seq(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, sb: S
         hip.current_stream_ptr(), x.data_ptr(), _rows(x), _dt(x), w.data_ptr(),
         state.data_ptr(), out.data_ptr(), C, sb.seq_of_t.data_ptr(), sb.cu_t.data_ptr(),
         sb.past_t.data_ptr(), sb.slots_t.data_ptr(), T, sb.num_seqs, C, taps,
-        int(add_input), int(act_silu), _dt(w))
+        int(add_input), int(act_silu), _dt(w), sb.max_chunk)
     hip.check(rc, "oa_causal_conv_seq")
     return out
 
@@ -236,55 +236,32 @@ def attention_biased_paged(q: torch.Tensor, gate_logits: torch.Tensor, k_cache: 
 
 def channel_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                        b_logits: torch.Tensor, a: torch.Tensor, dt_bias: torch.Tensor,
-                       a_log: torch.Tensor, state: torch.Tensor, sb: SeqBatch,
-                       H: int, G: int, D: int, Dv: int) -> torch.Tensor:
-    """Gated delta rule, one decay per head and key channel. q,k [T, G*D],
-    v [T, H*Dv] (after convolution and silu), b_logits [T,H], a [T,H*D] — all
-    may be column slices. state [slots,H,D,Dv] float32 is continued and
-    updated. Returns the read-out [T,H,Dv] float32."""
+                       a_log: torch.Tensor, norm_w: torch.Tensor, gate_logits: torch.Tensor,
+                       state: torch.Tensor, sb: SeqBatch, H: int, G: int, D: int, Dv: int,
+                       eps: float) -> torch.Tensor:
+    """Gated delta rule with one decay per head and key channel, through to
+    the gated read-out norm. q,k [T, G*D], v [T, H*Dv] (after convolution and
+    silu), b_logits [T,H], a [T,H*D], gate_logits [T,H*Dv] — all may be
+    column slices. state [slots,H,D,Dv] float32 is continued and updated.
+    Returns rms_norm_per_head(S^T q) * norm_w * sigmoid(gate) as [T, H*Dv]
+    in norm_w's type."""
     T = q.shape[0]
     if not q.is_cuda:
-        return torch_ref.channel_delta_rule(
+        o = torch_ref.channel_delta_rule(
             q.reshape(T, G, D), k.reshape(T, G, D), v.reshape(T, H, Dv), b_logits, a,
             dt_bias, a_log, state, sb.cu, sb.past, sb.slots)
+        return torch_ref.gated_head_rms_norm(o, norm_w, gate_logits, eps, norm_w.dtype)
     lib, hip = _lib()
-    dev = q.device
-    f32 = torch.float32
-    qn = torch.empty(T, G, D, dtype=f32, device=dev)
-    kn = torch.empty(T, G, D, dtype=f32, device=dev)
-    decay = torch.empty(T, H, D, dtype=f32, device=dev)
-    beta = torch.empty(T, H, dtype=f32, device=dev)
-    out = torch.empty(T, H, Dv, dtype=f32, device=dev)
-    dt = _dt(q)
-    assert state.dtype == f32 and state.is_contiguous() and state.shape[1:] == (H, D, Dv)
-    rc = lib.oa_delta_prepare(
+    out = torch.empty(T, H * Dv, dtype=norm_w.dtype, device=q.device)
+    assert state.dtype == torch.float32 and state.is_contiguous()
+    assert state.shape[1:] == (H, D, Dv)
+    rc = lib.oa_delta_rule_fused(
         hip.current_stream_ptr(), q.data_ptr(), _rows(q), k.data_ptr(), _rows(k),
-        b_logits.data_ptr(), _rows(b_logits), a.data_ptr(), _rows(a), dt_bias.data_ptr(),
-        a_log.data_ptr(), qn.data_ptr(), kn.data_ptr(), decay.data_ptr(), beta.data_ptr(),
-        T, H, G, D, dt)
-    hip.check(rc, "oa_delta_prepare")
-    rc = lib.oa_delta_recurrent(
-        hip.current_stream_ptr(), qn.data_ptr(), kn.data_ptr(), decay.data_ptr(),
-        beta.data_ptr(), v.data_ptr(), _rows(v), state.data_ptr(), out.data_ptr(),
-        sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.slots_t.data_ptr(), T, sb.num_seqs,
-        H, G, D, Dv, dt)
-    hip.check(rc, "oa_delta_recurrent")
-    return out
-
-
-def gated_head_rms_norm(o: torch.Tensor, w: torch.Tensor, gate_logits: torch.Tensor,
-                        eps: float) -> torch.Tensor:
-    """o [T,H,Dv] float32 -> per-head RMS norm * w[Dv] * sigmoid(gate_logits
-    [T, H*Dv]) in w's type, [T, H*Dv]."""
-    T, H, Dv = o.shape
-    if not o.is_cuda:
-        return torch_ref.gated_head_rms_norm(o, w, gate_logits, eps, w.dtype)
-    lib, hip = _lib()
-    out = torch.empty(T, H * Dv, dtype=w.dtype, device=o.device)
-    rc = lib.oa_gated_head_norm(
-        hip.current_stream_ptr(), o.data_ptr(), w.data_ptr(), gate_logits.data_ptr(),
-        _rows(gate_logits), out.data_ptr(), T, H, Dv, eps, _dt(w))
-    hip.check(rc, "oa_gated_head_norm")
+        v.data_ptr(), _rows(v), b_logits.data_ptr(), _rows(b_logits), a.data_ptr(), _rows(a),
+        dt_bias.data_ptr(), a_log.data_ptr(), norm_w.data_ptr(), gate_logits.data_ptr(),
+        _rows(gate_logits), state.data_ptr(), out.data_ptr(), sb.cu_t.data_ptr(),
+        sb.past_t.data_ptr(), sb.slots_t.data_ptr(), T, sb.num_seqs, H, G, D, Dv, eps, _dt(q))
+    hip.check(rc, "oa_delta_rule_fused")
     return out
 
 

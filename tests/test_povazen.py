@@ -45,7 +45,7 @@ def close(got, want, dtype, what=""):
     err = (got - want).pow(2).mean().sqrt() / (want.pow(2).mean().sqrt() + 1e-9)
     worst = (got - want).abs().max() / (want.abs().max() + 1e-9)
     if dtype == "fp32":
-        assert err < 5e-4 and worst < 2e-3, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
+        assert err < 1e-4 and worst < 1e-3, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
     else:
         assert err < 3e-2 and worst < 1.5e-1, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
 
@@ -381,7 +381,7 @@ def test_unequal_batch_equals_alone(mode, model_case):
     cfg, W = model_case
     eng = build_engine(cfg, W, dtype)
     Wr = rounded(W, dtype)
-    reqs = {"a": tokens_for(cfg, 53, 4), "b": tokens_for(cfg, 9, 5), "c": tokens_for(cfg, 1, 6),
+    reqs = {"a": tokens_for(cfg, 53, 4), "b": tokens_for(cfg, 9, 5), "c": tokens_for(cfg, 1, 7),
             "d": tokens_for(cfg, 30, 7)}
     plan = {"a": cut(reqs["a"], [11, 2, 1, 1, 19]), "b": cut(reqs["b"], [1]),
             "c": [reqs["c"]], "d": cut(reqs["d"], [2, 13, 1])}
