@@ -131,7 +131,8 @@ class ChannelDeltaMixer(nn.Module):
         return None
 
     def state_shapes(self) -> Dict[str, tuple]:
-        return {"conv": (self.taps - 1, self.n_conv), "S": (self.H, self.D, self.Dv)}
+        # S is kept column-major: [head, value column, key row]
+        return {"conv": (self.taps - 1, self.n_conv), "S": (self.H, self.Dv, self.D)}
 
     def forward(self, h, sb: mx.SeqBatch, kv, state) -> torch.Tensor:
         H, G, D, Dv = self.H, self.G, self.D, self.Dv

@@ -603,21 +603,32 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
 
 // ---------------------------------------------------------------------------
 // Gated delta rule with one decay per head and key channel, fused from the
-// convolved q/k/v to the gated, normed read-out. grid = (sequences, heads);
-// a block has one wave per 16 value columns. Lane = (column, row group): 16
-// columns x 4 row groups, each lane holds RPL consecutive key rows of its
-// column of S in registers (S lives in float32 in the state slot between
-// steps; a sequence that starts at position 0 starts from zero whatever
-// the slot holds).
+// convolved q/k/v to the gated, normed read-out. grid = (sequences, heads).
+// Lane = (row group, column): the 16 lanes of a DPP row split the D key rows
+// of one value column (RPL consecutive rows each), a wave holds 4 columns
+// per pass and P passes, a block all Dv columns of the head. S stays in
+// registers over the whole portion; between steps it lives in float32 in
+// the state slot as [H, Dv, D] (a column's rows contiguous). A sequence that
+// starts at position 0 starts from zero whatever the slot holds.
 // Per chunk of TCK tokens the block
 //   1. stages q, k (raw), decay = exp(-exp(A_log) softplus(a + dt_bias)),
 //      v and beta = sigmoid(b) in LDS as float32 (rows past D as zero),
 //   2. makes q and k unit vectors (q also times D^-1/2), a wave per token,
 //   3. runs the recurrence, every wave on its own columns:
 //        S <- decay * S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//      (the two column sums are DPP adds inside a 16-lane row),
 //   4. RMS-norms o over the head's value columns, times w, times
 //      sigmoid(gate), a wave per token, and stores it.
-template <int RPL, typename TC>
+__device__ __forceinline__ float row16_sum(float x) {
+    // all-reduce over the 16 lanes of a DPP row: quad swaps, then mirrors
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xF, 0xF, true));
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xF, 0xF, true));
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xF, 0xF, true));
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xF, 0xF, true));
+    return x;
+}
+
+template <int RPL, int P, typename TC>
 __global__ void delta_fused_kernel(
     const TC* __restrict__ q, int64_t qs, const TC* __restrict__ k, int64_t ks,
     const TC* __restrict__ v, int64_t vs, const TC* __restrict__ bl, int64_t bs,
@@ -626,7 +637,7 @@ __global__ void delta_fused_kernel(
     const TC* __restrict__ gate, int64_t gs, float* __restrict__ state,
     TC* __restrict__ out, const int* __restrict__ cu, const int* __restrict__ past,
     const int* __restrict__ slots, int H, int G, int D, int Dv, int TCK, float eps) {
-    constexpr int DP = RPL * 4;  // padded key size
+    constexpr int DP = RPL * 16;  // padded key size
     extern __shared__ float lds[];
     float* sq = lds;
     float* sk = sq + TCK * DP;
@@ -637,20 +648,24 @@ __global__ void delta_fused_kernel(
     const int b = blockIdx.x, h = blockIdx.y;
     const int tid = threadIdx.x, nth = blockDim.x;
     const int lane = tid & 63, wave = tid >> 6, nw = nth >> 6;
-    const int col = wave * 16 + (lane & 15), rg = lane >> 4;
-    const bool col_ok = col < Dv;
+    const int rg = lane & 15, cs = lane >> 4;
     const int lo = cu[b], n = cu[b + 1] - lo;
     if (n <= 0) return;
     const int kvh = h / (H / G);
-    float* st = state + (((int64_t)slots[b] * H + h) * D) * Dv;
+    float* st = state + (((int64_t)slots[b] * H + h) * Dv) * D;
     const float A = expf(ldf(a_log, h));
     const float qscale = 1.0f / sqrtf((float)D);
-    float S[RPL];
+    float S[P][RPL];
+    int col[P];
     const bool fresh = past[b] == 0;
 #pragma unroll
-    for (int i = 0; i < RPL; ++i) {
-        const int r = rg * RPL + i;
-        S[i] = (!fresh && col_ok && r < D) ? st[(int64_t)r * Dv + col] : 0.0f;
+    for (int p = 0; p < P; ++p) {
+        col[p] = (wave * P + p) * 4 + cs;
+#pragma unroll
+        for (int i = 0; i < RPL; ++i) {
+            const int r = rg * RPL + i;
+            S[p][i] = (!fresh && col[p] < Dv && r < D) ? st[(int64_t)col[p] * D + r] : 0.0f;
+        }
     }
     for (int c0 = 0; c0 < n; c0 += TCK) {
         const int nc = min(TCK, n - c0);
@@ -694,28 +709,41 @@ __global__ void delta_fused_kernel(
         __syncthreads();
         for (int tt = 0; tt < nc; ++tt) {
             const float bt = sb[tt];
-            const float vv = col_ok ? sv[tt * Dv + col] : 0.0f;
-            const float* kq = sk + tt * DP + rg * RPL;
-            const float* gq = sg + tt * DP + rg * RPL;
-            const float* qq = sq + tt * DP + rg * RPL;
-            float dot = 0.0f;
+            float kr[RPL], gr[RPL], qr[RPL];
 #pragma unroll
             for (int i = 0; i < RPL; ++i) {
-                S[i] *= gq[i];
-                dot += S[i] * kq[i];
+                kr[i] = sk[tt * DP + rg * RPL + i];
+                gr[i] = sg[tt * DP + rg * RPL + i];
+                qr[i] = sq[tt * DP + rg * RPL + i];
             }
-            dot += __shfl_xor(dot, 16, WAVE);
-            dot += __shfl_xor(dot, 32, WAVE);
-            const float u = bt * (vv - dot);
-            float o = 0.0f;
+            float dot[P], o[P];
 #pragma unroll
-            for (int i = 0; i < RPL; ++i) {
-                S[i] += kq[i] * u;
-                o += S[i] * qq[i];
+            for (int p = 0; p < P; ++p) {
+                dot[p] = 0.0f;
+#pragma unroll
+                for (int i = 0; i < RPL; ++i) {
+                    S[p][i] *= gr[i];
+                    dot[p] += S[p][i] * kr[i];
+                }
             }
-            o += __shfl_xor(o, 16, WAVE);
-            o += __shfl_xor(o, 32, WAVE);
-            if (rg == 0 && col_ok) so[tt * Dv + col] = o;
+#pragma unroll
+            for (int p = 0; p < P; ++p) dot[p] = row16_sum(dot[p]);
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                const float vv = col[p] < Dv ? sv[tt * Dv + col[p]] : 0.0f;
+                const float u = bt * (vv - dot[p]);
+                o[p] = 0.0f;
+#pragma unroll
+                for (int i = 0; i < RPL; ++i) {
+                    S[p][i] += kr[i] * u;
+                    o[p] += S[p][i] * qr[i];
+                }
+            }
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                o[p] = row16_sum(o[p]);
+                if (rg == 0 && col[p] < Dv) so[tt * Dv + col[p]] = o[p];
+            }
         }
         __syncthreads();
         for (int tt = wave; tt < nc; tt += nw) {
@@ -733,10 +761,12 @@ __global__ void delta_fused_kernel(
         // (which does) comes two barriers later
     }
 #pragma unroll
-    for (int i = 0; i < RPL; ++i) {
-        const int r = rg * RPL + i;
-        if (col_ok && r < D) st[(int64_t)r * Dv + col] = S[i];
-    }
+    for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int i = 0; i < RPL; ++i) {
+            const int r = rg * RPL + i;
+            if (col[p] < Dv && r < D) st[(int64_t)col[p] * D + r] = S[p][i];
+        }
 }
 
 // ---------------------------------------------------------------------------
@@ -989,17 +1019,17 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
     return 0;
 }
 
-template <int RPL>
+template <int RPL, int P>
 static int launch_delta(hipStream_t s, const void* q, int64_t qs, const void* k, int64_t ks,
                         const void* v, int64_t vs, const void* bl, int64_t bs, const void* a,
                         int64_t as, const void* dt_bias, const void* a_log, const void* norm_w,
                         const void* gate, int64_t gs, void* state, void* out, const void* cu,
                         const void* past, const void* slots, int B, int H, int G, int D, int Dv,
                         float eps, int dt) {
-    const int nw = CEIL_DIV(Dv, 16);
+    const int nw = CEIL_DIV(Dv, 4 * P);
     if (nw > 16) return -106;
     int tck = 16;
-    auto bytes = [&](int t) { return (size_t)(3 * t * RPL * 4 + 2 * t * Dv + t) * 4; };
+    auto bytes = [&](int t) { return (size_t)(3 * t * RPL * 16 + 2 * t * Dv + t) * 4; };
     while (tck > 2 && bytes(tck) > 60 * 1024) tck >>= 1;
     dim3 grid(B, H), blk(64 * nw);
 #define DARGS(TC)                                                                              \
@@ -1008,16 +1038,16 @@ static int launch_delta(hipStream_t s, const void* q, int64_t qs, const void* k,
         (float*)state, (TC*)out, (const int*)cu, (const int*)past, (const int*)slots, H, G, D,  \
         Dv, tck, eps
     if (dt == 1)
-        hipLaunchKernelGGL((delta_fused_kernel<RPL, float>), grid, blk, bytes(tck), s, DARGS(float));
+        hipLaunchKernelGGL((delta_fused_kernel<RPL, P, float>), grid, blk, bytes(tck), s, DARGS(float));
     else
-        hipLaunchKernelGGL((delta_fused_kernel<RPL, bf16s>), grid, blk, bytes(tck), s, DARGS(bf16s));
+        hipLaunchKernelGGL((delta_fused_kernel<RPL, P, bf16s>), grid, blk, bytes(tck), s, DARGS(bf16s));
 #undef DARGS
     HIP_CHECK_LAUNCH();
     return 0;
 }
 
 // q, k [T, G*D], v [T, H*Dv], bl [T, H], a [T, H*D], gate [T, H*Dv]: rows with
-// the given strides; out [T, H*Dv] contiguous.
+// the given strides; out [T, H*Dv] contiguous; state [slots, H, Dv, D].
 extern "C" int oa_delta_rule_fused(void* stream, const void* q, int64_t qs, const void* k,
                                    int64_t ks, const void* v, int64_t vs, const void* bl,
                                    int64_t bs, const void* a, int64_t as, const void* dt_bias,
@@ -1027,18 +1057,17 @@ extern "C" int oa_delta_rule_fused(void* stream, const void* q, int64_t qs, cons
                                    int D, int Dv, float eps, int dt) {
     if (T <= 0 || B <= 0) return 0;
     if (G < 1 || H % G != 0) return -100;
+    if (D > 256 || Dv > 256) return -105;
     hipStream_t s = (hipStream_t)stream;
-#define DL(R)                                                                                     \
-    launch_delta<R>(s, q, qs, k, ks, v, vs, bl, bs, a, as, dt_bias, a_log, norm_w, gate, gs, state, \
-                    out, cu, past, slots, B, H, G, D, Dv, eps, dt)
-    if (D <= 32) return DL(8);
-    if (D <= 64) return DL(16);
-    if (D <= 96) return DL(24);
-    if (D <= 128) return DL(32);
-    if (D <= 192) return DL(48);
-    if (D <= 256) return DL(64);
+#define DL(R, PP)                                                                                     \
+    launch_delta<R, PP>(s, q, qs, k, ks, v, vs, bl, bs, a, as, dt_bias, a_log, norm_w, gate, gs, state, \
+                        out, cu, past, slots, B, H, G, D, Dv, eps, dt)
+    const int r = D <= 64 ? 4 : (D <= 128 ? 8 : 16);
+    const int p = Dv <= 64 ? 1 : (Dv <= 128 ? 2 : 4);
+    if (r == 4) return p == 1 ? DL(4, 1) : (p == 2 ? DL(4, 2) : DL(4, 4));
+    if (r == 8) return p == 1 ? DL(8, 1) : (p == 2 ? DL(8, 2) : DL(8, 4));
+    return p == 1 ? DL(16, 1) : (p == 2 ? DL(16, 2) : DL(16, 4));
 #undef DL
-    return -105;
 }
 
 extern "C" int oa_softcap(void* stream, const void* x, void* out, int64_t n, float cap, int dt) {

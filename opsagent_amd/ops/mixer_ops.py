@@ -242,7 +242,8 @@ def channel_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     """Gated delta rule with one decay per head and key channel, through to
     the gated read-out norm. q,k [T, G*D], v [T, H*Dv] (after convolution and
     silu), b_logits [T,H], a [T,H*D], gate_logits [T,H*Dv] — all may be
-    column slices. state [slots,H,D,Dv] float32 is continued and updated.
+    column slices. state [slots,H,Dv,D] float32 (S transposed: a value
+    column's key rows contiguous) is continued and updated.
     Returns rms_norm_per_head(S^T q) * norm_w * sigmoid(gate) as [T, H*Dv]
     in norm_w's type."""
     T = q.shape[0]
@@ -254,7 +255,7 @@ def channel_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     lib, hip = _lib()
     out = torch.empty(T, H * Dv, dtype=norm_w.dtype, device=q.device)
     assert state.dtype == torch.float32 and state.is_contiguous()
-    assert state.shape[1:] == (H, D, Dv)
+    assert state.shape[1:] == (H, Dv, D)
     rc = lib.oa_delta_rule_fused(
         hip.current_stream_ptr(), q.data_ptr(), _rows(q), k.data_ptr(), _rows(k),
         v.data_ptr(), _rows(v), b_logits.data_ptr(), _rows(b_logits), a.data_ptr(), _rows(a),

@@ -289,8 +289,8 @@ def attention_biased_paged(q, gate_logits, k_cache, v_cache, cu, past, block_tab
 
 def channel_delta_rule(q, k, v, b_logits, a, dt_bias, a_log, state, cu, past, slots):
     """Gated delta rule with a decay per head and key channel, continued from
-    `state` [slots, H, D, Dv] float32 (zero at position 0 whatever the slot
-    holds). q,k [T,G,D], v [T,H,Dv] after convolution and silu; b_logits
+    `state` [slots, H, Dv, D] float32 (S stored transposed; zero at position 0
+    whatever the slot holds). q,k [T,G,D], v [T,H,Dv] after convolution and silu; b_logits
     [T,H]; a [T,H*D]. Returns the read-out [T,H,Dv] float32; updates state."""
     T, G, D = q.shape
     H, Dv = v.shape[1], v.shape[2]
@@ -309,13 +309,15 @@ def channel_delta_rule(q, k, v, b_logits, a, dt_bias, a_log, state, cu, past, sl
         lo, hi = cu[bi], cu[bi + 1]
         if hi == lo:
             continue
-        S = state[slots[bi]].clone() if past[bi] > 0 else torch.zeros_like(state[slots[bi]])
+        S = state[slots[bi]].transpose(-1, -2).clone()
+        if past[bi] == 0:
+            S.zero_()
         for t in range(lo, hi):
             S = S * g[t].unsqueeze(-1)
             u = beta[t].unsqueeze(-1) * (vf[t] - torch.einsum("hdv,hd->hv", S, kf[t]))
             S = S + kf[t].unsqueeze(-1) * u.unsqueeze(1)
             out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
-        state[slots[bi]] = S
+        state[slots[bi]] = S.transpose(-1, -2)
     return out
 
 
