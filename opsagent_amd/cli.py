@@ -222,6 +222,24 @@ def serve(
     )
 
 
+@app.command(context_settings={"allow_extra_args": True, "ignore_unknown_options": True})
+def replay(
+    ctx: typer.Context,
+    model: str = typer.Option(..., "--model", help="checkpoint folder (config.json + model.safetensors)"),
+    dtype: str = typer.Option("bfloat16", "--dtype", help="bfloat16 | float32"),
+    out: str = typer.Option(..., "--out", help="folder for <step>.f32 logits"),
+    max_tokens: int = typer.Option(..., "--max-tokens", help="tokens live requests hold at most"),
+):
+    """Replay a token-id trace (JSON steps on stdin) through the engine and
+    write the wanted logits; samples nothing (same as bin/trace_run)."""
+    from opsagent_amd.engine.replay import main as replay_main
+
+    raise typer.Exit(replay_main(
+        ["--model", model, "--dtype", dtype, "--out", out, "--max-tokens", str(max_tokens)]
+        + list(ctx.args)
+    ))
+
+
 @app.command()
 def version():
     """Print version (ref version.go:29-41)."""

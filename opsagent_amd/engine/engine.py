@@ -253,7 +253,7 @@ class LLMEngine:
             self.model = LlamaForCausalLM(self.spec, self.dtype, self.device, self.seed)
         self.model.eval()
         weights = str(cfg.get("weights", "") or "")
-        if not weights:
+        if weights in ("", "random"):
             # a checkpoint folder brings its own weights
             weights = getattr(self.spec, "weights_path", None) or "random"
         if weights not in ("random", ""):

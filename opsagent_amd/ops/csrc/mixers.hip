@@ -28,6 +28,29 @@ __device__ __forceinline__ float ldf(const bf16s* p, int64_t i) { return bf16_to
 __device__ __forceinline__ void stf(float* p, int64_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void stf(bf16s* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
 
+// 8 consecutive elements at once (16-byte aligned for bf16, 32 for float32)
+__device__ __forceinline__ void ld8(const float* p, int64_t i, float* o) {
+    const float4 a = *reinterpret_cast<const float4*>(p + i);
+    const float4 b = *reinterpret_cast<const float4*>(p + i + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+__device__ __forceinline__ void ld8(const bf16s* p, int64_t i, float* o) {
+    const uint4 a = *reinterpret_cast<const uint4*>(p + i);
+    o[0] = bf16_lo(a.x); o[1] = bf16_hi(a.x); o[2] = bf16_lo(a.y); o[3] = bf16_hi(a.y);
+    o[4] = bf16_lo(a.z); o[5] = bf16_hi(a.z); o[6] = bf16_lo(a.w); o[7] = bf16_hi(a.w);
+}
+__device__ __forceinline__ void st8(float* p, int64_t i, const float* v) {
+    *reinterpret_cast<float4*>(p + i) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void st8(bf16s* p, int64_t i, const float* v) {
+    uint4 a;
+    a.x = pack_bf16x2(v[0], v[1]); a.y = pack_bf16x2(v[2], v[3]);
+    a.z = pack_bf16x2(v[4], v[5]); a.w = pack_bf16x2(v[6], v[7]);
+    *reinterpret_cast<uint4*>(p + i) = a;
+}
+
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float softplusf_(float z) {
     return fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z)));
@@ -66,6 +89,53 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
         if (add_input) acc += ldf(x, (int64_t)t * xs + c);
         if (act_silu) acc = acc * sigmoidf_(acc);
         stf(out, (int64_t)t * os + c, acc);
+    }
+}
+
+// The same with 8 channels per thread (C, row strides multiples of 8).
+template <int TAPS, typename TI, typename TW, typename TO>
+__global__ __launch_bounds__(256) void causal_conv_vec_kernel(
+    const TI* __restrict__ x, int64_t xs, const TW* __restrict__ w,
+    const float* __restrict__ state, TO* __restrict__ out, int64_t os,
+    const int* __restrict__ seq_of, const int* __restrict__ cu,
+    const int* __restrict__ past, const int* __restrict__ slots, int T, int C,
+    int taps_rt, int add_input, int act_silu) {
+    constexpr int taps = TAPS;
+    const int C8 = C / 8;
+    const int64_t total = (int64_t)T * C8;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int t = (int)(idx / C8), c = (int)(idx % C8) * 8;
+        const int b = seq_of[t];
+        const int lo = cu[b];
+        const int local = t - lo;
+        const int pos = past[b] + local;
+        const float* st = state + (int64_t)slots[b] * (taps - 1) * C;
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float xv[8];
+        float wv[TAPS][8];   // the 8 channels' weights: 8*TAPS consecutive values
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) ld8(w, (int64_t)c * taps + 8 * j, wv[j]);
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+            const int d = j - (taps - 1);
+            if (pos + d < 0) continue;
+            const int s = local + d;
+            if (s >= 0) ld8(x, (int64_t)(lo + s) * xs + c, xv);
+            else ld8(st, (int64_t)(taps - 1 + s) * C + c, xv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += wv[(e * TAPS + j) / 8][(e * TAPS + j) % 8] * xv[e];
+        }
+        if (add_input) {
+            ld8(x, (int64_t)t * xs + c, xv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += xv[e];
+        }
+        if (act_silu) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = acc[e] * sigmoidf_(acc[e]);
+        }
+        st8(out, (int64_t)t * os + c, acc);
     }
 }
 
@@ -167,6 +237,53 @@ __global__ __launch_bounds__(256) void group_rmsnorm_kernel(
                 residual[(int64_t)t * C + c] = v;
             }
             if (copy) stf(copy, (int64_t)t * C + c, v);
+        }
+    }
+}
+
+// The same with 8 elements per lane and the part held in registers between
+// the two passes (part size a multiple of 8, at most 64*8*GN_IT).
+#define GN_IT 4
+template <typename TY, typename TW, typename TO>
+__global__ __launch_bounds__(256) void group_rmsnorm_vec_kernel(
+    const TY* __restrict__ y, int64_t ys, const TW* __restrict__ w,
+    float* __restrict__ residual, TO* __restrict__ copy, int C, int groups,
+    float eps) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int gs = C / groups;
+    for (int g = wave; g < groups; g += nw) {
+        const int64_t base = (int64_t)t * ys + (int64_t)g * gs;
+        float v[GN_IT][8];
+        float ss = 0.0f;
+#pragma unroll
+        for (int it = 0; it < GN_IT; ++it) {
+            const int i = (it * 64 + lane) * 8;
+            if (i < gs) {
+                ld8(y, base + i, v[it]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += v[it][e] * v[it][e];
+            }
+        }
+        ss = wave_reduce_sum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)gs + eps);
+#pragma unroll
+        for (int it = 0; it < GN_IT; ++it) {
+            const int i = (it * 64 + lane) * 8;
+            if (i < gs) {
+                const int c = g * gs + i;
+                float wv[8], rv[8];
+                ld8(w, c, wv);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[it][e] = v[it][e] * r * wv[e];
+                if (residual) {
+                    ld8(residual, (int64_t)t * C + c, rv);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[it][e] += rv[e];
+                    st8(residual, (int64_t)t * C + c, v[it]);
+                }
+                if (copy) st8(copy, (int64_t)t * C + c, v[it]);
+            }
         }
     }
 }
@@ -395,12 +512,20 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
 // Scores, the distance penalty, softmax statistics and weights are float32;
 // a weight enters the value product as a bf16 pair hi + lo (two MFMAs), so
 // it keeps 16 bits of mantissa.
-// LDS: K tile [64][D+4], V tile transposed [Dv][64+4] (bf16).
+// LDS: K tile [64][D+8], V tile transposed [Dv][64+4] (bf16).
+// Where the key size divides by 32 (QK32) and always for the value product,
+// the gfx950 form v_mfma_f32_16x16x32_bf16 is used: same i/j mapping, a lane
+// holds k = 8*(lane>>4)..+7. The value product feeds it the weights a lane
+// already holds (keys 16*mt + 4*(lane>>4) + r of two adjacent 16-key tiles)
+// and reads V^T at the same keys, so no lane exchange is needed: the sum
+// over k does not care about the order of the keys.
 typedef short s4_t __attribute__((ext_vector_type(4)));
+typedef short s8_t __attribute__((ext_vector_type(8)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 #define MF_KT 64
+#define MF_KPAD 8
 
-template <int MAXD, int MAXDV>
+template <int MAXD, int MAXDV, bool QK32>
 __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const bf16s* __restrict__ q, const bf16s* __restrict__ gate, int64_t gs,
     const bf16s* __restrict__ k_cache, const bf16s* __restrict__ v_cache,
@@ -410,8 +535,8 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const float* __restrict__ slopes, int B, int H, int G, int D, int Dv, int HB,
     float scale, int nsplit) {
     extern __shared__ float lds[];
-    bf16s* Ks = (bf16s*)lds;                        // [64][D+4]
-    const int kst = D + 4;
+    bf16s* Ks = (bf16s*)lds;                        // [64][D+8]
+    const int kst = D + MF_KPAD;
     bf16s* Vt = Ks + (size_t)MF_KT * kst;           // [Dv][68]
     const int vst = MF_KT + 4;
     const int R = H / G;
@@ -440,14 +565,25 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int* bt = block_table + (int64_t)b * max_blocks;
     const float slope = slopes[h];
 
-    s4_t qf[MAXD];
+    s4_t qf[QK32 ? 1 : MAXD];
+    s8_t qf8[QK32 ? MAXD / 2 : 1];
     {
         const int tk = lo + t0 + min(lc, max(ntok - 1, 0));
-        const bf16s* qr = q + ((int64_t)tk * H + h) * D + 4 * lg;
+        const bf16s* qr = q + ((int64_t)tk * H + h) * D;
+        if (QK32) {
 #pragma unroll
-        for (int ks = 0; ks < MAXD; ++ks) {
-            if (16 * ks < D && ntok > 0) qf[ks] = *reinterpret_cast<const s4_t*>(qr + 16 * ks);
-            else qf[ks] = s4_t{0, 0, 0, 0};
+            for (int ks = 0; ks < MAXD / 2; ++ks) {
+                if (32 * ks < D && ntok > 0)
+                    qf8[ks] = *reinterpret_cast<const s8_t*>(qr + 32 * ks + 8 * lg);
+                else qf8[ks] = s8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < MAXD; ++ks) {
+                if (16 * ks < D && ntok > 0)
+                    qf[ks] = *reinterpret_cast<const s4_t*>(qr + 16 * ks + 4 * lg);
+                else qf[ks] = s4_t{0, 0, 0, 0};
+            }
         }
     }
     f4_t o[MAXDV];
@@ -495,12 +631,22 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
             sc[mt] = f4_t{0.f, 0.f, 0.f, 0.f};
-            const bf16s* kr = Ks + (16 * mt + lc) * kst + 4 * lg;
+            const bf16s* kr = Ks + (16 * mt + lc) * kst;
+            if (QK32) {
 #pragma unroll
-            for (int ks = 0; ks < MAXD; ++ks)
-                if (16 * ks < D)
-                    sc[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
-                        *reinterpret_cast<const s4_t*>(kr + 16 * ks), qf[ks], sc[mt], 0, 0, 0);
+                for (int ks = 0; ks < MAXD / 2; ++ks)
+                    if (32 * ks < D)
+                        sc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            *reinterpret_cast<const s8_t*>(kr + 32 * ks + 8 * lg), qf8[ks], sc[mt],
+                            0, 0, 0);
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < MAXD; ++ks)
+                    if (16 * ks < D)
+                        sc[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                            *reinterpret_cast<const s4_t*>(kr + 16 * ks + 4 * lg), qf[ks], sc[mt],
+                            0, 0, 0);
+            }
         }
         float mloc = -INFINITY;
 #pragma unroll
@@ -540,10 +686,14 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
                 o[dt] *= corr;
                 const bf16s* vr = Vt + (16 * dt + lc) * vst + 4 * lg;
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt) {
-                    const s4_t a = *reinterpret_cast<const s4_t*>(vr + 16 * mt);
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, phi[mt], o[dt], 0, 0, 0);
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, plo[mt], o[dt], 0, 0, 0);
+                for (int kb = 0; kb < 2; ++kb) {
+                    const s4_t a0 = *reinterpret_cast<const s4_t*>(vr + 32 * kb);
+                    const s4_t a1 = *reinterpret_cast<const s4_t*>(vr + 32 * kb + 16);
+                    const s8_t a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+                    const s8_t bh = __builtin_shufflevector(phi[2 * kb], phi[2 * kb + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    const s8_t bl = __builtin_shufflevector(plo[2 * kb], plo[2 * kb + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bh, o[dt], 0, 0, 0);
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bl, o[dt], 0, 0, 0);
                 }
             }
         }
@@ -574,30 +724,53 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     }
 }
 
-// merge key-split partials: one wave per (token, head)
+// merge key-split partials: one wave per (token, head); lanes first take
+// one split each for the statistics, then one value channel each
 template <typename TC>
 __global__ __launch_bounds__(64) void attn_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
     const TC* __restrict__ gate, int64_t gs, TC* __restrict__ out, int H, int Dv,
     int nsplit) {
+    __shared__ float wsh[64];
     const int64_t row = blockIdx.x;  // tok * H + h
     const int tok = (int)(row / H), h = (int)(row % H);
     const int lane = threadIdx.x;
-    float mx = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part_ml[(row * nsplit + s) * 2]);
-    float l = 0.0f;
-    for (int s = 0; s < nsplit; ++s) {
-        const float ms = part_ml[(row * nsplit + s) * 2];
-        if (ms != -INFINITY) l += part_ml[(row * nsplit + s) * 2 + 1] * expf(ms - mx);
+    float mx = -INFINITY, lsum = 0.0f;
+    for (int s0 = 0; s0 < nsplit; s0 += 64) {          // running merge over groups of 64 splits
+        const int s = s0 + lane;
+        const float ms = s < nsplit ? part_ml[(row * nsplit + s) * 2] : -INFINITY;
+        const float ls = s < nsplit ? part_ml[(row * nsplit + s) * 2 + 1] : 0.0f;
+        const float gmx = fmaxf(mx, wave_reduce_max(ms));
+        const float wgt = (ms == -INFINITY) ? 0.0f : expf(ms - gmx);
+        lsum = lsum * ((mx == -INFINITY) ? 0.0f : expf(mx - gmx)) + wave_reduce_sum(ls * wgt);
+        mx = gmx;
     }
-    const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) / l;
-    for (int ch = lane; ch < Dv; ch += 64) {
-        float a = 0.0f;
-        for (int s = 0; s < nsplit; ++s) {
-            const float ms = part_ml[(row * nsplit + s) * 2];
-            if (ms != -INFINITY) a += part_o[(row * nsplit + s) * Dv + ch] * expf(ms - mx);
+    const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) / lsum;
+    float acc[ATT_MAXV];
+#pragma unroll
+    for (int c = 0; c < ATT_MAXV; ++c) acc[c] = 0.0f;
+    for (int s0 = 0; s0 < nsplit; s0 += 64) {
+        const int s = s0 + lane;
+        const float ms = s < nsplit ? part_ml[(row * nsplit + s) * 2] : -INFINITY;
+        __syncthreads();
+        wsh[lane] = (ms == -INFINITY) ? 0.0f : expf(ms - mx);
+        __syncthreads();
+        const int ns = min(64, nsplit - s0);
+#pragma unroll 4
+        for (int j = 0; j < ns; ++j) {
+            const float wj = wsh[j];
+            const float* po = part_o + (row * nsplit + s0 + j) * Dv;
+#pragma unroll
+            for (int c = 0; c < ATT_MAXV; ++c) {
+                const int ch = lane + 64 * c;
+                if (ch < Dv) acc[c] += po[ch] * wj;
+            }
         }
-        stf(out, row * Dv + ch, a * gt);
+    }
+#pragma unroll
+    for (int c = 0; c < ATT_MAXV; ++c) {
+        const int ch = lane + 64 * c;
+        if (ch < Dv) stf(out, row * Dv + ch, acc[c] * gt);
     }
 }
 
@@ -658,13 +831,27 @@ __global__ void delta_fused_kernel(
     float S[P][RPL];
     int col[P];
     const bool fresh = past[b] == 0;
+    const bool vec4 = (D & 3) == 0;   // a lane's rows of a column are 16-byte pieces
 #pragma unroll
     for (int p = 0; p < P; ++p) {
         col[p] = (wave * P + p) * 4 + cs;
+        const bool live = !fresh && col[p] < Dv;
 #pragma unroll
-        for (int i = 0; i < RPL; ++i) {
-            const int r = rg * RPL + i;
-            S[p][i] = (!fresh && col[p] < Dv && r < D) ? st[(int64_t)col[p] * D + r] : 0.0f;
+        for (int i4 = 0; i4 < RPL / 4; ++i4) {
+            const int r = rg * RPL + 4 * i4;
+            float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (live && vec4 && r < D) {
+                x = *reinterpret_cast<const float4*>(st + (int64_t)col[p] * D + r);
+            } else if (live) {
+                if (r < D) x.x = st[(int64_t)col[p] * D + r];
+                if (r + 1 < D) x.y = st[(int64_t)col[p] * D + r + 1];
+                if (r + 2 < D) x.z = st[(int64_t)col[p] * D + r + 2];
+                if (r + 3 < D) x.w = st[(int64_t)col[p] * D + r + 3];
+            }
+            S[p][4 * i4] = x.x;
+            S[p][4 * i4 + 1] = x.y;
+            S[p][4 * i4 + 2] = x.z;
+            S[p][4 * i4 + 3] = x.w;
         }
     }
     for (int c0 = 0; c0 < n; c0 += TCK) {
@@ -761,12 +948,22 @@ __global__ void delta_fused_kernel(
         // (which does) comes two barriers later
     }
 #pragma unroll
-    for (int p = 0; p < P; ++p)
+    for (int p = 0; p < P; ++p) {
+        if (col[p] >= Dv) continue;
 #pragma unroll
-        for (int i = 0; i < RPL; ++i) {
-            const int r = rg * RPL + i;
-            if (col[p] < Dv && r < D) st[(int64_t)col[p] * D + r] = S[p][i];
+        for (int i4 = 0; i4 < RPL / 4; ++i4) {
+            const int r = rg * RPL + 4 * i4;
+            float* dst = st + (int64_t)col[p] * D + r;
+            if (vec4 && r < D) {
+                *reinterpret_cast<float4*>(dst) =
+                    make_float4(S[p][4 * i4], S[p][4 * i4 + 1], S[p][4 * i4 + 2], S[p][4 * i4 + 3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (r + e < D) dst[e] = S[p][4 * i4 + e];
+            }
         }
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -845,7 +1042,30 @@ extern "C" int oa_causal_conv_seq(void* stream, const void* x, int64_t xs, int x
     (const TI*)x, xs, (const TW*)w, (const float*)state, (TW*)out, os,             \
         (const int*)seq_of, (const int*)cu, (const int*)past, (const int*)slots, T, \
         C, taps, add_input, act_silu
-    if (x_dt == 1 && dt == 1)
+    const bool vec = C % 8 == 0 && xs % 8 == 0 && os % 8 == 0 && taps >= 2 && taps <= 4 &&
+                     ((uintptr_t)x % 32 == 0) && ((uintptr_t)out % 16 == 0) &&
+                     ((uintptr_t)w % 32 == 0);
+    if (vec) {
+        dim3 gv(grid_for((int64_t)T * (C / 8)));
+#define CV(TP)                                                                                        \
+    do {                                                                                              \
+        if (x_dt == 1 && dt == 1)                                                                     \
+            hipLaunchKernelGGL((causal_conv_vec_kernel<TP, float, float, float>), gv, blk, 0, s,      \
+                               CONV_ARGS(float, float));                                              \
+        else if (x_dt == 1 && dt == 0)                                                                \
+            hipLaunchKernelGGL((causal_conv_vec_kernel<TP, float, bf16s, bf16s>), gv, blk, 0, s,      \
+                               CONV_ARGS(float, bf16s));                                              \
+        else if (x_dt == 0 && dt == 0)                                                                \
+            hipLaunchKernelGGL((causal_conv_vec_kernel<TP, bf16s, bf16s, bf16s>), gv, blk, 0, s,      \
+                               CONV_ARGS(bf16s, bf16s));                                              \
+        else                                                                                          \
+            return -101;                                                                              \
+    } while (0)
+        if (taps == 2) CV(2);
+        else if (taps == 3) CV(3);
+        else CV(4);
+#undef CV
+    } else if (x_dt == 1 && dt == 1)
         hipLaunchKernelGGL((causal_conv_kernel<float, float, float>), g1, blk, 0, s, CONV_ARGS(float, float));
     else if (x_dt == 1 && dt == 0)
         hipLaunchKernelGGL((causal_conv_kernel<float, bf16s, bf16s>), g1, blk, 0, s, CONV_ARGS(float, bf16s));
@@ -876,7 +1096,17 @@ extern "C" int oa_group_rmsnorm(void* stream, const void* y, int64_t ys, int y_d
     hipStream_t s = (hipStream_t)stream;
     dim3 g(T), blk(256);
 #define GN_ARGS(TY, TW) (const TY*)y, ys, (const TW*)w, (float*)residual, (TW*)copy, C, groups, eps
-    if (y_dt == 1 && dt == 1)
+    const int gsz = C / groups;
+    if (gsz % 8 == 0 && gsz <= 64 * 8 * GN_IT && ys % 8 == 0 && (uintptr_t)y % 32 == 0) {
+        if (y_dt == 1 && dt == 1)
+            hipLaunchKernelGGL((group_rmsnorm_vec_kernel<float, float, float>), g, blk, 0, s, GN_ARGS(float, float));
+        else if (y_dt == 1 && dt == 0)
+            hipLaunchKernelGGL((group_rmsnorm_vec_kernel<float, bf16s, bf16s>), g, blk, 0, s, GN_ARGS(float, bf16s));
+        else if (y_dt == 0 && dt == 0)
+            hipLaunchKernelGGL((group_rmsnorm_vec_kernel<bf16s, bf16s, bf16s>), g, blk, 0, s, GN_ARGS(bf16s, bf16s));
+        else
+            return -101;
+    } else if (y_dt == 1 && dt == 1)
         hipLaunchKernelGGL((group_rmsnorm_kernel<float, float, float>), g, blk, 0, s, GN_ARGS(float, float));
     else if (y_dt == 1 && dt == 0)
         hipLaunchKernelGGL((group_rmsnorm_kernel<float, bf16s, bf16s>), g, blk, 0, s, GN_ARGS(float, bf16s));
@@ -923,8 +1153,8 @@ extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int* T
     if (attn_path(H, G, D, Dv, dt)) {
         *TQ = 16 * (4 / attn_hb(R));
         *KT = MF_KT;
-        *kstride = D + 4;
-        *lds_bytes = (MF_KT * (D + 4) + Dv * (MF_KT + 4)) * 2;
+        *kstride = D + MF_KPAD;
+        *lds_bytes = (MF_KT * (D + MF_KPAD) + Dv * (MF_KT + 4)) * 2;
         return 0;
     }
     if (R > 4 * ATT_MAXR) return -102;
@@ -943,7 +1173,7 @@ extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int* T
     return -103;
 }
 
-template <int MAXD, int MAXDV>
+template <int MAXD, int MAXDV, bool QK32>
 static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void* q, const void* gate,
                              int64_t gs, const void* k_cache, const void* v_cache, void* out,
                              void* part_o, void* part_ml, const void* cu, const void* past,
@@ -951,9 +1181,9 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                              const void* slopes, int B, int H, int G, int D, int Dv, int HB,
                              float scale, int nsplit) {
     if (lds_bytes > 48 * 1024)
-        (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV>,
+        (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV, QK32>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    hipLaunchKernelGGL((attn_bias_mfma_kernel<MAXD, MAXDV>), grid, dim3(256), lds_bytes, s,
+    hipLaunchKernelGGL((attn_bias_mfma_kernel<MAXD, MAXDV, QK32>), grid, dim3(256), lds_bytes, s,
                        (const bf16s*)q, (const bf16s*)gate, gs, (const bf16s*)k_cache,
                        (const bf16s*)v_cache, (bf16s*)out, (float*)part_o, (float*)part_ml,
                        (const int*)cu, (const int*)past, (const int*)block_table, max_blocks,
@@ -976,9 +1206,17 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
     if (attn_path(H, G, D, Dv, dt)) {
         const int R = H / G, HB = attn_hb(R);
         dim3 grid(ntiles, G * (R / HB), nsplit);
-#define MF(A, Bv) launch_attn_mfma<A, Bv>(s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out, part_o, \
-                                          part_ml, cu, past, block_table, max_blocks, block_size, slopes, \
-                                          B, H, G, D, Dv, HB, scale, nsplit)
+#define MF(A, Bv)                                                                                   \
+    do {                                                                                            \
+        if (D % 32 == 0)                                                                            \
+            launch_attn_mfma<A, Bv, true>(s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out,   \
+                                          part_o, part_ml, cu, past, block_table, max_blocks,       \
+                                          block_size, slopes, B, H, G, D, Dv, HB, scale, nsplit);   \
+        else                                                                                        \
+            launch_attn_mfma<A, Bv, false>(s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out,  \
+                                           part_o, part_ml, cu, past, block_table, max_blocks,      \
+                                           block_size, slopes, B, H, G, D, Dv, HB, scale, nsplit);  \
+    } while (0)
         const int a = D <= 64 ? 4 : (D <= 128 ? 8 : 16), bv = Dv <= 64 ? 4 : (Dv <= 128 ? 8 : 16);
         if (a == 4 && bv == 4) MF(4, 4);
         else if (a == 4 && bv == 8) MF(4, 8);
