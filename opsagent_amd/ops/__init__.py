@@ -769,10 +769,11 @@ def greedy_sample_masked(
         assert logits.is_contiguous()
         if mask_bits is not None:
             assert mask_bits.dtype == torch.int32 and mask_bits.is_contiguous()
+        ws32 = torch.empty(B * 16 * 2, dtype=torch.int32, device=logits.device)
         rc = lib.oa_masked_argmax_f32(
             hip.current_stream_ptr(), logits.data_ptr(),
             mask_bits.data_ptr() if mask_bits is not None else None,
-            out.data_ptr(), B, V,
+            ws32.data_ptr(), out.data_ptr(), B, V,
         )
         hip.check(rc, "oa_masked_argmax_f32")
         return out

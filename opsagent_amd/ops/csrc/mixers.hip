@@ -351,6 +351,91 @@ __global__ __launch_bounds__(256) void attn_prepare_kernel(
     }
 }
 
+// The same with 8 elements per thread (all sizes and strides multiples of 8).
+template <typename TC>
+__global__ __launch_bounds__(256) void attn_prepare_vec_kernel(
+    const TC* __restrict__ qkv, int64_t qs, const TC* __restrict__ bias,
+    const TC* __restrict__ qw, const TC* __restrict__ kw, TC* __restrict__ q_out,
+    TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+    const int* __restrict__ slot_mapping, const int* __restrict__ cu, int B, int H,
+    int G, int D, int Dv, float eps) {
+    __shared__ float red[8];
+    const int t = blockIdx.x;
+    if (t >= cu[B]) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const TC* row = qkv + (int64_t)t * qs;
+    const int nq = H * D, nk = G * D;
+    const int64_t slot = slot_mapping[t];
+    auto val8 = [&](int i, float* o) {
+        ld8(row, i, o);
+        if (bias) {
+            float bv[8];
+            ld8(bias, i, bv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] += bv[e];
+        }
+    };
+    float sq = 0.0f, sk = 0.0f, x[8], wv[8];
+    for (int i = threadIdx.x * 8; i < nq; i += blockDim.x * 8) {
+        val8(i, x);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq += x[e] * x[e];
+    }
+    for (int i = threadIdx.x * 8; i < nk; i += blockDim.x * 8) {
+        val8(nq + i, x);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sk += x[e] * x[e];
+    }
+    sq = wave_reduce_sum(sq);
+    sk = wave_reduce_sum(sk);
+    if (lane == 0) {
+        red[wave] = sq;
+        red[4 + wave] = sk;
+    }
+    __syncthreads();
+    sq = 0.0f;
+    sk = 0.0f;
+    for (int i = 0; i < nw; ++i) {
+        sq += red[i];
+        sk += red[4 + i];
+    }
+    const float rq = 1.0f / sqrtf(sq / (float)nq + eps);
+    const float rk = 1.0f / sqrtf(sk / (float)nk + eps);
+    for (int i = threadIdx.x * 8; i < nq; i += blockDim.x * 8) {
+        val8(i, x);
+        ld8(qw, i, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= rq * wv[e];
+        st8(q_out, (int64_t)t * nq + i, x);
+    }
+    for (int i = threadIdx.x * 8; i < nk; i += blockDim.x * 8) {
+        val8(nq + i, x);
+        ld8(kw, i, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= rk * wv[e];
+        st8(k_cache, slot * nk + i, x);
+    }
+    // value heads: 8 lanes... a 16-lane group per head pass keeps it simple:
+    // each wave takes heads wave, wave+nw, ...; lanes take 8 channels each
+    for (int g = wave; g < G; g += nw) {
+        const int off = nq + nk + g * Dv;
+        float sv = 0.0f;
+        for (int i = lane * 8; i < Dv; i += 64 * 8) {
+            val8(off + i, x);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sv += x[e] * x[e];
+        }
+        sv = wave_reduce_sum(sv);
+        const float rv = 1.0f / sqrtf(sv / (float)Dv + eps);
+        for (int i = lane * 8; i < Dv; i += 64 * 8) {
+            val8(off + i, x);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] *= rv;
+            st8(v_cache, slot * (int64_t)(G * Dv) + g * Dv + i, x);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Softmax attention with a linear distance penalty over the paged cache.
 //   score(i, j) = q_i . k_j * scale - slope_h * (i - j),  j <= i
@@ -563,7 +648,10 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int wave_last = pb + t0 + ntok - 1;
     const int block_last = pb + min(n, tile * TQ + TQ) - 1;
     const int* bt = block_table + (int64_t)b * max_blocks;
-    const float slope = slopes[h];
+    // softmax in the exp2 domain: log2(e) folded into the scale and the slope
+    const float LOG2E = 1.4426950408889634f;
+    const float slope = slopes[h] * LOG2E;
+    const float scale2 = scale * LOG2E;
 
     s4_t qf[QK32 ? 1 : MAXD];
     s8_t qf8[QK32 ? MAXD / 2 : 1];
@@ -593,28 +681,40 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
 
     const int nkt = block_last / MF_KT + 1;
     const int dch = D / 8, vch = Dv / 8;
+    // pages are a power of two: shifts, not divisions, in the staging loops
+    const int bsh = 31 - __clz(block_size), bmask = block_size - 1;
+    const int kj0 = threadIdx.x / dch, kc0 = threadIdx.x % dch;
+    const int kjs = 256 / dch, kcs = 256 % dch;
     for (int kt = split; kt < nkt; kt += nsplit) {
         const int k0 = kt * MF_KT;
         const int nk = min(MF_KT, block_last + 1 - k0);
         __syncthreads();
-        for (int i = threadIdx.x; i < MF_KT * dch; i += 256) {
-            const int j = i / dch, c = i % dch;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (j < nk) {
-                const int key = k0 + j;
-                const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
-                v = *reinterpret_cast<const uint4*>(k_cache + (slot * G + g) * D + 8 * c);
+        {   // K rows: (key j, 8-wide piece c) walks forward by 256 pieces per step
+            int j = kj0, c = kc0;
+            for (int i = threadIdx.x; i < MF_KT * dch; i += 256) {
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (j < nk) {
+                    const int key = k0 + j;
+                    const int64_t slot = ((int64_t)bt[key >> bsh] << bsh) + (key & bmask);
+                    v = *reinterpret_cast<const uint4*>(k_cache + (slot * G + g) * D + 8 * c);
+                }
+                uint2* dst = reinterpret_cast<uint2*>(Ks + j * kst + 8 * c);
+                dst[0] = make_uint2(v.x, v.y);
+                dst[1] = make_uint2(v.z, v.w);
+                j += kjs;
+                c += kcs;
+                if (c >= dch) {
+                    c -= dch;
+                    ++j;
+                }
             }
-            uint2* dst = reinterpret_cast<uint2*>(Ks + j * kst + 8 * c);
-            dst[0] = make_uint2(v.x, v.y);
-            dst[1] = make_uint2(v.z, v.w);
         }
         for (int i = threadIdx.x; i < MF_KT * vch; i += 256) {
             const int j = i % MF_KT, c = i / MF_KT;   // lanes along keys: adjacent LDS columns
             uint4 v = make_uint4(0, 0, 0, 0);
             if (j < nk) {
                 const int key = k0 + j;
-                const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
+                const int64_t slot = ((int64_t)bt[key >> bsh] << bsh) + (key & bmask);
                 v = *reinterpret_cast<const uint4*>(v_cache + (slot * G + g) * Dv + 8 * c);
             }
             const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -654,7 +754,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = k0 + 16 * mt + 4 * lg + r;
-                float v = sc[mt][r] * scale - slope * (float)(pos - key);
+                float v = sc[mt][r] * scale2 - slope * (float)(pos - key);
                 v = (key <= pos) ? v : -INFINITY;
                 sc[mt][r] = v;
                 mloc = fmaxf(mloc, v);
@@ -662,19 +762,22 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
         const float mnew = fmaxf(m, mloc);
-        const float corr = (m == -INFINITY) ? 0.0f : expf(m - mnew);
+        // v_exp_f32 gives 0 for -inf, so masked keys need no select; only a
+        // row that has seen no key yet (m = mnew = -inf) must be kept off NaN
+        const float msub = (mnew == -INFINITY) ? 0.0f : mnew;
+        const float corr = __builtin_amdgcn_exp2f(m - msub);
         float lsum = 0.0f;
         s4_t phi[4], plo[4];
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float v = sc[mt][r];
-                const float p = (v == -INFINITY) ? 0.0f : expf(v - mnew);
+                const float p = __builtin_amdgcn_exp2f(sc[mt][r] - msub);
                 lsum += p;
-                const bf16s hi = f32_to_bf16(p);
-                phi[mt][r] = (short)hi;
-                plo[mt][r] = (short)f32_to_bf16(p - bf16_to_f32(hi));
+                // hi = p truncated to bf16 (exact remainder), lo = remainder rounded
+                const uint32_t pu = __float_as_uint(p);
+                phi[mt][r] = (short)(pu >> 16);
+                plo[mt][r] = (short)f32_to_bf16(p - __uint_as_float(pu & 0xffff0000u));
             }
         lsum += __shfl_xor(lsum, 16, WAVE);
         lsum += __shfl_xor(lsum, 32, WAVE);
@@ -718,7 +821,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
             if (16 * dt < Dv)
                 *reinterpret_cast<f4_t*>(part_o + pr * Dv + 16 * dt + 4 * lg) = o[dt];
         if (lg == 0) {
-            part_ml[pr * 2] = m;
+            part_ml[pr * 2] = m * 0.6931471805599453f;   // back to the natural-log domain
             part_ml[pr * 2 + 1] = l;
         }
     }
@@ -1125,6 +1228,21 @@ extern "C" int oa_attn_prepare(void* stream, const void* qkv, int64_t qs, const 
                                int G, int D, int Dv, float eps, int dt) {
     if (T <= 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    if (D % 8 == 0 && Dv % 8 == 0 && qs % 8 == 0 && (uintptr_t)qkv % 32 == 0 &&
+        (!bias || (uintptr_t)bias % 32 == 0)) {
+        if (dt == 1)
+            hipLaunchKernelGGL((attn_prepare_vec_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)qkv,
+                               qs, (const float*)bias, (const float*)qw, (const float*)kw, (float*)q_out,
+                               (float*)k_cache, (float*)v_cache, (const int*)slot_mapping, (const int*)cu,
+                               B, H, G, D, Dv, eps);
+        else
+            hipLaunchKernelGGL((attn_prepare_vec_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const bf16s*)qkv,
+                               qs, (const bf16s*)bias, (const bf16s*)qw, (const bf16s*)kw, (bf16s*)q_out,
+                               (bf16s*)k_cache, (bf16s*)v_cache, (const int*)slot_mapping, (const int*)cu,
+                               B, H, G, D, Dv, eps);
+        HIP_CHECK_LAUNCH();
+        return 0;
+    }
     if (dt == 1)
         hipLaunchKernelGGL((attn_prepare_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)qkv, qs,
                            (const float*)bias, (const float*)qw, (const float*)kw, (float*)q_out, (float*)k_cache,

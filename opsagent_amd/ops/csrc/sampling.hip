@@ -119,17 +119,26 @@ extern "C" int oa_masked_argmax(void* stream, const void* logits, const void* ma
     return 0;
 }
 
-// float32 logits (models whose head emits float32, any V): one block per
-// row scans the whole row; lowest index wins ties, -1 if nothing is allowed.
-__global__ __launch_bounds__(256) void masked_argmax_f32_kernel(
+// float32 logits (models whose head emits float32, any V): grid (chunks, B);
+// each block scans its part of the row and leaves its best (value, index)
+// in ws[b][chunk]; a second small kernel picks among the chunks. Lowest
+// index wins ties, -1 if nothing is allowed. No atomics, nothing to clear.
+#define F32_CHUNKS 16
+__device__ __forceinline__ bool better_f32(float v, int i, float bv, int bi) {
+    return i >= 0 && (bi < 0 || v > bv || (v == bv && i < bi));
+}
+
+__global__ __launch_bounds__(256) void masked_argmax_f32_scan(
     const float* __restrict__ logits, const uint32_t* __restrict__ mask,
-    int* __restrict__ out, int V, int mask_words) {
-    const int b = blockIdx.x;
+    float* __restrict__ ws_val, int* __restrict__ ws_idx, int V, int mask_words) {
+    const int b = blockIdx.y, chunk = blockIdx.x;
     const float* row = logits + (size_t)b * V;
     const uint32_t* mrow = mask ? mask + (size_t)b * mask_words : nullptr;
+    const int per = CEIL_DIV(V, F32_CHUNKS);
+    const int t0 = chunk * per, t1 = min(V, t0 + per);
     float best = -INFINITY;
     int besti = -1;
-    for (int t = threadIdx.x; t < V; t += blockDim.x) {
+    for (int t = t0 + threadIdx.x; t < t1; t += blockDim.x) {
         if (mrow && !((mrow[t >> 5] >> (t & 31)) & 1u)) continue;
         const float v = row[t];
         if (besti < 0 || v > best) {  // ascending t per thread: first max kept
@@ -139,9 +148,9 @@ __global__ __launch_bounds__(256) void masked_argmax_f32_kernel(
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
-        float ov = __shfl_xor(best, off, WAVE);
-        int oi = __shfl_xor(besti, off, WAVE);
-        if (oi >= 0 && (besti < 0 || ov > best || (ov == best && oi < besti))) {
+        const float ov = __shfl_xor(best, off, WAVE);
+        const int oi = __shfl_xor(besti, off, WAVE);
+        if (better_f32(ov, oi, best, besti)) {
             best = ov;
             besti = oi;
         }
@@ -156,20 +165,43 @@ __global__ __launch_bounds__(256) void masked_argmax_f32_kernel(
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int w = 1; w < 4; ++w)
-            if (si[w] >= 0 && (besti < 0 || sv[w] > best || (sv[w] == best && si[w] < besti))) {
+            if (better_f32(sv[w], si[w], best, besti)) {
                 best = sv[w];
                 besti = si[w];
             }
-        out[b] = besti;
+        ws_val[b * F32_CHUNKS + chunk] = best;
+        ws_idx[b * F32_CHUNKS + chunk] = besti;
     }
 }
 
+__global__ void masked_argmax_f32_finish(const float* __restrict__ ws_val,
+                                         const int* __restrict__ ws_idx,
+                                         int* __restrict__ out, int B) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= B) return;
+    float best = -INFINITY;
+    int besti = -1;
+    for (int c = 0; c < F32_CHUNKS; ++c)
+        if (better_f32(ws_val[b * F32_CHUNKS + c], ws_idx[b * F32_CHUNKS + c], best, besti)) {
+            best = ws_val[b * F32_CHUNKS + c];
+            besti = ws_idx[b * F32_CHUNKS + c];
+        }
+    out[b] = besti;
+}
+
+// ws: B * F32_CHUNKS * 8 bytes of scratch
 extern "C" int oa_masked_argmax_f32(void* stream, const void* logits, const void* mask,
-                                    void* out, int B, int V) {
+                                    void* ws, void* out, int B, int V) {
     if (B <= 0) return 0;
-    hipLaunchKernelGGL(masked_argmax_f32_kernel, dim3(B), dim3(256), 0,
+    float* ws_val = (float*)ws;
+    int* ws_idx = (int*)ws + (size_t)B * F32_CHUNKS;
+    hipLaunchKernelGGL(masked_argmax_f32_scan, dim3(F32_CHUNKS, B), dim3(256), 0,
                        (hipStream_t)stream, (const float*)logits, (const uint32_t*)mask,
-                       (int*)out, V, CEIL_DIV(V, 32));
+                       ws_val, ws_idx, V, CEIL_DIV(V, 32));
+    HIP_CHECK_LAUNCH();
+    hipLaunchKernelGGL(masked_argmax_f32_finish, dim3(CEIL_DIV(B, 64)), dim3(64), 0,
+                       (hipStream_t)stream, (const float*)ws_val, (const int*)ws_idx,
+                       (int*)out, B);
     HIP_CHECK_LAUNCH();
     return 0;
 }

@@ -53,7 +53,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.oa_gemv_gateup_ex.restype = i
     lib.oa_masked_argmax.argtypes = [p, p, p, p, p, i, i]
     lib.oa_masked_argmax.restype = i
-    lib.oa_masked_argmax_f32.argtypes = [p, p, p, p, i, i]
+    lib.oa_masked_argmax_f32.argtypes = [p, p, p, p, p, i, i]
     lib.oa_masked_argmax_f32.restype = i
     lib.oa_attention_prefill.argtypes = [p, p, p, p, p, i, i, i, i, i, i, f, i, i, i]
     lib.oa_attention_prefill.restype = i

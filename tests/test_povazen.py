@@ -554,3 +554,34 @@ def test_decode_graph_equals_eager(dtype, model_case):
             assert any(e["graph"] is not None for e in eng._graphs.values())
     for i in reqs:
         assert torch.equal(outs[0][i], outs[1][i]), f"graph replay differs for {i}"
+
+
+@gpu
+@pytest.mark.parametrize("V", [97, 2048, 32003])
+def test_float32_masked_argmax(V):
+    """The sampler's float32 path: ties go to the lowest index, masked
+    tokens never win, an all-masked row gives -1."""
+    from opsagent_amd import ops
+
+    g = torch.Generator().manual_seed(V)
+    B = 5
+    logits = torch.randn(B, V, generator=g)
+    logits[1, 40] = logits[1, 7] = logits[1].max() + 1         # tie: index 7 wins
+    allow = torch.rand(B, V, generator=g) > 0.5
+    allow[2] = False                                           # nothing allowed
+    allow[3] = True
+    words = (V + 31) // 32
+    bits = torch.zeros(B, words * 32, dtype=torch.bool)
+    bits[:, :V] = allow
+    packed = (bits.view(B, words, 32).long() << torch.arange(32)).sum(-1)
+    packed = torch.where(packed >= 2 ** 31, packed - 2 ** 32, packed).to(torch.int32)
+    got = ops.greedy_sample_masked(logits.cuda(), packed.cuda()).cpu().tolist()
+    for b in range(B):
+        if not allow[b].any():
+            assert got[b] == -1
+        else:
+            want = int(logits[b].masked_fill(~allow[b], float("-inf")).argmax())
+            assert logits[b, got[b]] == logits[b, want] and allow[b, got[b]]
+            assert got[b] == int((logits[b].masked_fill(~allow[b], float("-inf")) == logits[b, want]).nonzero()[0])
+    free = ops.greedy_sample_masked(logits.cuda(), None).cpu().tolist()
+    assert free[1] == 7
