@@ -911,8 +911,9 @@ __global__ void delta_fused_kernel(
     const TC* __restrict__ a, int64_t as, const TC* __restrict__ dt_bias,
     const TC* __restrict__ a_log, const TC* __restrict__ norm_w,
     const TC* __restrict__ gate, int64_t gs, float* __restrict__ state,
-    TC* __restrict__ out, const int* __restrict__ cu, const int* __restrict__ past,
-    const int* __restrict__ slots, int H, int G, int D, int Dv, int TCK, float eps) {
+    TC* __restrict__ out, float* __restrict__ o_raw, const int* __restrict__ cu,
+    const int* __restrict__ past, const int* __restrict__ slots, int H, int G, int D,
+    int Dv, int TCK, float eps) {
     constexpr int DP = RPL * 16;  // padded key size
     extern __shared__ float lds[];
     float* sq = lds;
@@ -935,9 +936,14 @@ __global__ void delta_fused_kernel(
     int col[P];
     const bool fresh = past[b] == 0;
     const bool vec4 = (D & 3) == 0;   // a lane's rows of a column are 16-byte pieces
+    // gridDim.z > 1: the head's value columns are split over blocks (few
+    // (sequence, head) pairs, long portions); the read-out then goes to
+    // o_raw and the head norm runs as its own launch
+    const int cpb = Dv / gridDim.z, cb = blockIdx.z * cpb, cend = cb + cpb;
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-        col[p] = (wave * P + p) * 4 + cs;
+        col[p] = cb + (wave * P + p) * 4 + cs;
+        if (col[p] >= cend) col[p] = Dv;              // past this block's share: idle
         const bool live = !fresh && col[p] < Dv;
 #pragma unroll
         for (int i4 = 0; i4 < RPL / 4; ++i4) {
@@ -1036,6 +1042,14 @@ __global__ void delta_fused_kernel(
             }
         }
         __syncthreads();
+        if (gridDim.z > 1) {
+            for (int i = tid; i < nc * cpb; i += nth) {
+                const int tt = i / cpb, c = cb + i % cpb;
+                o_raw[((int64_t)(tb + tt) * H + h) * Dv + c] = so[tt * Dv + c];
+            }
+            __syncthreads();   // `so` is rewritten by the next chunk's recurrence
+            continue;
+        }
         for (int tt = wave; tt < nc; tt += nw) {
             float ss = 0.0f;
             for (int c = lane; c < Dv; c += 64) ss += so[tt * Dv + c] * so[tt * Dv + c];
@@ -1065,6 +1079,29 @@ __global__ void delta_fused_kernel(
                 for (int e = 0; e < 4; ++e)
                     if (r + e < D) dst[e] = S[p][4 * i4 + e];
             }
+        }
+    }
+}
+
+// per-head RMS norm of a float32 read-out, times w[Dv], times sigmoid(gate):
+// one block per token, one wave per head (used when the delta rule's columns
+// were split over blocks)
+template <typename TC>
+__global__ __launch_bounds__(256) void gated_head_norm_kernel(
+    const float* __restrict__ o, const TC* __restrict__ w,
+    const TC* __restrict__ gate, int64_t gs, TC* __restrict__ out, int H, int Dv,
+    float eps) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    for (int h = wave; h < H; h += nw) {
+        const float* src = o + ((int64_t)t * H + h) * Dv;
+        float ss = 0.0f;
+        for (int i = lane; i < Dv; i += 64) ss += src[i] * src[i];
+        ss = wave_reduce_sum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
+        for (int i = lane; i < Dv; i += 64) {
+            const float gt = sigmoidf_(ldf(gate, (int64_t)t * gs + h * Dv + i));
+            stf(out, ((int64_t)t * H + h) * Dv + i, src[i] * r * ldf(w, i) * gt);
         }
     }
 }
@@ -1379,20 +1416,20 @@ template <int RPL, int P>
 static int launch_delta(hipStream_t s, const void* q, int64_t qs, const void* k, int64_t ks,
                         const void* v, int64_t vs, const void* bl, int64_t bs, const void* a,
                         int64_t as, const void* dt_bias, const void* a_log, const void* norm_w,
-                        const void* gate, int64_t gs, void* state, void* out, const void* cu,
-                        const void* past, const void* slots, int B, int H, int G, int D, int Dv,
-                        float eps, int dt) {
-    const int nw = CEIL_DIV(Dv, 4 * P);
+                        const void* gate, int64_t gs, void* state, void* out, void* o_raw,
+                        const void* cu, const void* past, const void* slots, int B, int H, int G,
+                        int D, int Dv, float eps, int dt, int csplit) {
+    const int nw = CEIL_DIV(Dv / csplit, 4 * P);
     if (nw > 16) return -106;
     int tck = 16;
     auto bytes = [&](int t) { return (size_t)(3 * t * RPL * 16 + 2 * t * Dv + t) * 4; };
     while (tck > 2 && bytes(tck) > 60 * 1024) tck >>= 1;
-    dim3 grid(B, H), blk(64 * nw);
+    dim3 grid(B, H, csplit), blk(64 * nw);
 #define DARGS(TC)                                                                              \
     (const TC*)q, qs, (const TC*)k, ks, (const TC*)v, vs, (const TC*)bl, bs, (const TC*)a, as,  \
         (const TC*)dt_bias, (const TC*)a_log, (const TC*)norm_w, (const TC*)gate, gs,           \
-        (float*)state, (TC*)out, (const int*)cu, (const int*)past, (const int*)slots, H, G, D,  \
-        Dv, tck, eps
+        (float*)state, (TC*)out, (float*)o_raw, (const int*)cu, (const int*)past,               \
+        (const int*)slots, H, G, D, Dv, tck, eps
     if (dt == 1)
         hipLaunchKernelGGL((delta_fused_kernel<RPL, P, float>), grid, blk, bytes(tck), s, DARGS(float));
     else
@@ -1404,26 +1441,41 @@ static int launch_delta(hipStream_t s, const void* q, int64_t qs, const void* k,
 
 // q, k [T, G*D], v [T, H*Dv], bl [T, H], a [T, H*D], gate [T, H*Dv]: rows with
 // the given strides; out [T, H*Dv] contiguous; state [slots, H, Dv, D].
+// csplit > 1 splits each head's value columns over that many blocks (Dv must
+// divide by 4*csplit) and needs o_raw, float32 [T, H*Dv].
 extern "C" int oa_delta_rule_fused(void* stream, const void* q, int64_t qs, const void* k,
                                    int64_t ks, const void* v, int64_t vs, const void* bl,
                                    int64_t bs, const void* a, int64_t as, const void* dt_bias,
                                    const void* a_log, const void* norm_w, const void* gate,
-                                   int64_t gs, void* state, void* out, const void* cu,
-                                   const void* past, const void* slots, int T, int B, int H, int G,
-                                   int D, int Dv, float eps, int dt) {
+                                   int64_t gs, void* state, void* out, void* o_raw,
+                                   const void* cu, const void* past, const void* slots, int T,
+                                   int B, int H, int G, int D, int Dv, float eps, int dt,
+                                   int csplit) {
     if (T <= 0 || B <= 0) return 0;
     if (G < 1 || H % G != 0) return -100;
     if (D > 256 || Dv > 256) return -105;
+    if (csplit < 1 || Dv % (4 * csplit) != 0 || (csplit > 1 && !o_raw)) return -107;
     hipStream_t s = (hipStream_t)stream;
 #define DL(R, PP)                                                                                     \
     launch_delta<R, PP>(s, q, qs, k, ks, v, vs, bl, bs, a, as, dt_bias, a_log, norm_w, gate, gs, state, \
-                        out, cu, past, slots, B, H, G, D, Dv, eps, dt)
+                        out, o_raw, cu, past, slots, B, H, G, D, Dv, eps, dt, csplit)
     const int r = D <= 64 ? 4 : (D <= 128 ? 8 : 16);
-    const int p = Dv <= 64 ? 1 : (Dv <= 128 ? 2 : 4);
-    if (r == 4) return p == 1 ? DL(4, 1) : (p == 2 ? DL(4, 2) : DL(4, 4));
-    if (r == 8) return p == 1 ? DL(8, 1) : (p == 2 ? DL(8, 2) : DL(8, 4));
-    return p == 1 ? DL(16, 1) : (p == 2 ? DL(16, 2) : DL(16, 4));
+    const int cpb = Dv / csplit;
+    const int p = cpb <= 64 ? 1 : (cpb <= 128 ? 2 : 4);
+    int rc;
+    if (r == 4) rc = p == 1 ? DL(4, 1) : (p == 2 ? DL(4, 2) : DL(4, 4));
+    else if (r == 8) rc = p == 1 ? DL(8, 1) : (p == 2 ? DL(8, 2) : DL(8, 4));
+    else rc = p == 1 ? DL(16, 1) : (p == 2 ? DL(16, 2) : DL(16, 4));
 #undef DL
+    if (rc || csplit == 1) return rc;
+    if (dt == 1)
+        hipLaunchKernelGGL((gated_head_norm_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)o_raw,
+                           (const float*)norm_w, (const float*)gate, gs, (float*)out, H, Dv, eps);
+    else
+        hipLaunchKernelGGL((gated_head_norm_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const float*)o_raw,
+                           (const bf16s*)norm_w, (const bf16s*)gate, gs, (bf16s*)out, H, Dv, eps);
+    HIP_CHECK_LAUNCH();
+    return 0;
 }
 
 extern "C" int oa_softcap(void* stream, const void* x, void* out, int64_t n, float cap, int dt) {

@@ -125,7 +125,7 @@ def _declare_mixers(lib: ctypes.CDLL) -> None:
         "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p,
                                i, i, i, i, i, i, i, f, i, i],
         "oa_delta_rule_fused": [p, p, i64, p, i64, p, i64, p, i64, p, i64, p, p, p, p, i64,
-                                p, p, p, p, p, i, i, i, i, i, i, f, i],
+                                p, p, p, p, p, p, i, i, i, i, i, i, f, i, i],
         "oa_softcap": [p, p, p, i64, f, i],
         "oa_silu_mul_rows": [p, p, p, i64, i, i],
         "oa_embed_rows": [p, p, p, p, i, i, i],

@@ -256,12 +256,26 @@ def channel_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     out = torch.empty(T, H * Dv, dtype=norm_w.dtype, device=q.device)
     assert state.dtype == torch.float32 and state.is_contiguous()
     assert state.shape[1:] == (H, Dv, D)
+    # one block per (sequence, head) runs the recurrence of ALL value columns
+    # on one CU; long portions of few sequences split the columns over blocks
+    # instead (the head norm then runs as its own launch on a float32 buffer)
+    csplit, o_raw = 1, None
+    pairs = sb.num_seqs * H
+    if sb.max_chunk >= 64 and pairs < 192:
+        for c in (8, 4, 2):
+            if Dv % (4 * c) == 0 and Dv // c >= 16 and pairs * c <= 512:
+                csplit = c
+                break
+    if csplit > 1:
+        o_raw = torch.empty(T, H * Dv, dtype=torch.float32, device=q.device)
     rc = lib.oa_delta_rule_fused(
         hip.current_stream_ptr(), q.data_ptr(), _rows(q), k.data_ptr(), _rows(k),
         v.data_ptr(), _rows(v), b_logits.data_ptr(), _rows(b_logits), a.data_ptr(), _rows(a),
         dt_bias.data_ptr(), a_log.data_ptr(), norm_w.data_ptr(), gate_logits.data_ptr(),
-        _rows(gate_logits), state.data_ptr(), out.data_ptr(), sb.cu_t.data_ptr(),
-        sb.past_t.data_ptr(), sb.slots_t.data_ptr(), T, sb.num_seqs, H, G, D, Dv, eps, _dt(q))
+        _rows(gate_logits), state.data_ptr(), out.data_ptr(),
+        o_raw.data_ptr() if o_raw is not None else None, sb.cu_t.data_ptr(),
+        sb.past_t.data_ptr(), sb.slots_t.data_ptr(), T, sb.num_seqs, H, G, D, Dv, eps, _dt(q),
+        csplit)
     hip.check(rc, "oa_delta_rule_fused")
     return out
 

@@ -230,18 +230,25 @@ def test_attention_mixer_alone(mode, geom):
         close(torch.cat(outs, 0), want, dtype, f"attention {sizes}")
 
 
+# (heads, kv_heads, dim, vdim): the last two are wide enough for the kernel
+# to split a head's value columns over several blocks on long portions
+DELTA_GEOMS = [(4, 2, 20, 24), (2, 1, 32, 64), (2, 2, 64, 128)]
+
+
 @pytest.mark.parametrize("mode", MODES)
-def test_delta_mixer_alone(mode):
+@pytest.mark.parametrize("geom", DELTA_GEOMS)
+def test_delta_mixer_alone(mode, geom):
     device, dtype = mode
     _skip_if_wrong_device(device)
-    cfg, W, eng = _single_layer("D", dtype, device, conv=4)
+    dh, dk, dd, dv = geom
+    cfg, W, eng = _single_layer("D", dtype, device, conv=4, d_heads=dh, d_kv=dk, d_dim=dd, d_vdim=dv)
     mixer = eng.model.layers[0].mixer
     g = torch.Generator().manual_seed(6)
-    T = 41
+    T = 150
     h = torch.randn(T, cfg["width"], generator=g).to(tdtype(dtype))
     want = O.channel_delta_mixer(h.double(), {k: v.double() for k, v in W.items()}, "l0.mix.",
                                  cfg["layers"][0]["mixer"], cfg["norm"]["eps"])
-    for slot, sizes in ((0, [T]), (2, [3, 2, 17, 1, 1, 1, 16])):
+    for slot, sizes in ((0, [T]), (2, [3, 2, 17, 1, 1, 1, 16, 70, 39]), (1, [80, 1, 69])):
         for t in eng.state_pool.tensors[0].values():
             t.fill_(3.0)                                 # a used slot
         outs, at = [], 0
