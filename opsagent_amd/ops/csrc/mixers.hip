@@ -610,7 +610,7 @@ typedef float f4_t __attribute__((ext_vector_type(4)));
 #define MF_KT 64
 #define MF_KPAD 8
 
-template <int MAXD, int MAXDV, bool QK32>
+template <int MAXD, int MAXDV, bool QK32, int NT>
 __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const bf16s* __restrict__ q, const bf16s* __restrict__ gate, int64_t gs,
     const bf16s* __restrict__ k_cache, const bf16s* __restrict__ v_cache,
@@ -619,13 +619,15 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int* __restrict__ block_table, int max_blocks, int block_size,
     const float* __restrict__ slopes, int B, int H, int G, int D, int Dv, int HB,
     float scale, int nsplit) {
+    // NT: 16-token sub-tiles per wave. Every K and V fragment read from LDS
+    // feeds NT MFMAs, and a staged tile serves NT times the query rows.
     extern __shared__ float lds[];
     bf16s* Ks = (bf16s*)lds;                        // [64][D+8]
     const int kst = D + MF_KPAD;
     bf16s* Vt = Ks + (size_t)MF_KT * kst;           // [Dv][68]
     const int vst = MF_KT + 4;
     const int R = H / G;
-    const int TT = 4 / HB, TQ = 16 * TT;
+    const int TT = 4 / HB, TQ = 16 * TT * NT;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lc = lane & 15, lg = lane >> 4;
     const int hgroups = R / HB;
@@ -642,10 +644,15 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     }
     if (b >= B) return;
     const int pb = past[b];
-    const int t0 = tile * TQ + (wave / HB) * 16;    // this wave's first local token
-    const int ntok = max(0, min(16, n - t0));
-    const int pos = pb + t0 + lc;                   // this lane's token position
-    const int wave_last = pb + t0 + ntok - 1;
+    const int t0 = tile * TQ + (wave / HB) * 16 * NT;   // this wave's first local token
+    int ntok[NT], pos[NT];
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+        ntok[u] = max(0, min(16, n - (t0 + 16 * u)));
+        pos[u] = pb + t0 + 16 * u + lc;                  // this lane's token position
+    }
+    const int wave_ntok = max(0, min(16 * NT, n - t0));
+    const int wave_last = pb + t0 + wave_ntok - 1;
     const int block_last = pb + min(n, tile * TQ + TQ) - 1;
     const int* bt = block_table + (int64_t)b * max_blocks;
     // softmax in the exp2 domain: log2(e) folded into the scale and the slope
@@ -653,31 +660,37 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const float slope = slopes[h] * LOG2E;
     const float scale2 = scale * LOG2E;
 
-    s4_t qf[QK32 ? 1 : MAXD];
-    s8_t qf8[QK32 ? MAXD / 2 : 1];
-    {
-        const int tk = lo + t0 + min(lc, max(ntok - 1, 0));
-        const bf16s* qr = q + ((int64_t)tk * H + h) * D;
+    s4_t qf[NT][QK32 ? 1 : MAXD];
+    s8_t qf8[NT][QK32 ? MAXD / 2 : 1];
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+        const int tk = lo + t0 + 16 * u + min(lc, max(ntok[u] - 1, 0));
+        const bf16s* qr = q + ((int64_t)min(tk, lo + n - 1) * H + h) * D;
         if (QK32) {
 #pragma unroll
             for (int ks = 0; ks < MAXD / 2; ++ks) {
-                if (32 * ks < D && ntok > 0)
-                    qf8[ks] = *reinterpret_cast<const s8_t*>(qr + 32 * ks + 8 * lg);
-                else qf8[ks] = s8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                if (32 * ks < D && ntok[u] > 0)
+                    qf8[u][ks] = *reinterpret_cast<const s8_t*>(qr + 32 * ks + 8 * lg);
+                else qf8[u][ks] = s8_t{0, 0, 0, 0, 0, 0, 0, 0};
             }
         } else {
 #pragma unroll
             for (int ks = 0; ks < MAXD; ++ks) {
-                if (16 * ks < D && ntok > 0)
-                    qf[ks] = *reinterpret_cast<const s4_t*>(qr + 16 * ks + 4 * lg);
-                else qf[ks] = s4_t{0, 0, 0, 0};
+                if (16 * ks < D && ntok[u] > 0)
+                    qf[u][ks] = *reinterpret_cast<const s4_t*>(qr + 16 * ks + 4 * lg);
+                else qf[u][ks] = s4_t{0, 0, 0, 0};
             }
         }
     }
-    f4_t o[MAXDV];
+    f4_t o[NT][MAXDV];
+    float m[NT], l[NT];
 #pragma unroll
-    for (int i = 0; i < MAXDV; ++i) o[i] = f4_t{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.0f;
+    for (int u = 0; u < NT; ++u) {
+        m[u] = -INFINITY;
+        l[u] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < MAXDV; ++i) o[u][i] = f4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     const int nkt = block_last / MF_KT + 1;
     const int dch = D / 8, vch = Dv / 8;
@@ -698,9 +711,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
                     const int64_t slot = ((int64_t)bt[key >> bsh] << bsh) + (key & bmask);
                     v = *reinterpret_cast<const uint4*>(k_cache + (slot * G + g) * D + 8 * c);
                 }
-                uint2* dst = reinterpret_cast<uint2*>(Ks + j * kst + 8 * c);
-                dst[0] = make_uint2(v.x, v.y);
-                dst[1] = make_uint2(v.z, v.w);
+                *reinterpret_cast<uint4*>(Ks + j * kst + 8 * c) = v;
                 j += kjs;
                 c += kcs;
                 if (c >= dch) {
@@ -725,104 +736,124 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
             }
         }
         __syncthreads();
-        if (ntok <= 0 || k0 > wave_last) continue;
-        // S^T tiles: keys k0 + 16*mt + 4*lg + r, token lc
-        f4_t sc[4];
+        if (wave_ntok <= 0 || k0 > wave_last) continue;
+        // S^T tiles: keys k0 + 16*mt + 4*lg + r, token lc of sub-tile u
+        f4_t sc[NT][4];
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
-            sc[mt] = f4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < NT; ++u) sc[u][mt] = f4_t{0.f, 0.f, 0.f, 0.f};
             const bf16s* kr = Ks + (16 * mt + lc) * kst;
             if (QK32) {
 #pragma unroll
                 for (int ks = 0; ks < MAXD / 2; ++ks)
-                    if (32 * ks < D)
-                        sc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            *reinterpret_cast<const s8_t*>(kr + 32 * ks + 8 * lg), qf8[ks], sc[mt],
-                            0, 0, 0);
+                    if (32 * ks < D) {
+                        const s8_t kf = *reinterpret_cast<const s8_t*>(kr + 32 * ks + 8 * lg);
+#pragma unroll
+                        for (int u = 0; u < NT; ++u)
+                            sc[u][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf8[u][ks],
+                                                                               sc[u][mt], 0, 0, 0);
+                    }
             } else {
 #pragma unroll
                 for (int ks = 0; ks < MAXD; ++ks)
-                    if (16 * ks < D)
-                        sc[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
-                            *reinterpret_cast<const s4_t*>(kr + 16 * ks + 4 * lg), qf[ks], sc[mt],
-                            0, 0, 0);
+                    if (16 * ks < D) {
+                        const s4_t kf = *reinterpret_cast<const s4_t*>(kr + 16 * ks + 4 * lg);
+#pragma unroll
+                        for (int u = 0; u < NT; ++u)
+                            sc[u][mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf, qf[u][ks],
+                                                                                 sc[u][mt], 0, 0, 0);
+                    }
             }
         }
-        float mloc = -INFINITY;
+        s4_t phi[NT][4], plo[NT][4];
+        float corr[NT];
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+        for (int u = 0; u < NT; ++u) {
+            float mloc = -INFINITY;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = k0 + 16 * mt + 4 * lg + r;
-                float v = sc[mt][r] * scale2 - slope * (float)(pos - key);
-                v = (key <= pos) ? v : -INFINITY;
-                sc[mt][r] = v;
-                mloc = fmaxf(mloc, v);
-            }
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
-        const float mnew = fmaxf(m, mloc);
-        // v_exp_f32 gives 0 for -inf, so masked keys need no select; only a
-        // row that has seen no key yet (m = mnew = -inf) must be kept off NaN
-        const float msub = (mnew == -INFINITY) ? 0.0f : mnew;
-        const float corr = __builtin_amdgcn_exp2f(m - msub);
-        float lsum = 0.0f;
-        s4_t phi[4], plo[4];
+            for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+                for (int r = 0; r < 4; ++r) {
+                    const int key = k0 + 16 * mt + 4 * lg + r;
+                    float v = sc[u][mt][r] * scale2 - slope * (float)(pos[u] - key);
+                    v = (key <= pos[u]) ? v : -INFINITY;
+                    sc[u][mt][r] = v;
+                    mloc = fmaxf(mloc, v);
+                }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, WAVE));
+            const float mnew = fmaxf(m[u], mloc);
+            // v_exp_f32 gives 0 for -inf, so masked keys need no select; only a
+            // row that has seen no key yet (m = mnew = -inf) must be kept off NaN
+            const float msub = (mnew == -INFINITY) ? 0.0f : mnew;
+            corr[u] = __builtin_amdgcn_exp2f(m[u] - msub);
+            float lsum = 0.0f;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float p = __builtin_amdgcn_exp2f(sc[mt][r] - msub);
-                lsum += p;
-                // hi = p truncated to bf16 (exact remainder), lo = remainder rounded
-                const uint32_t pu = __float_as_uint(p);
-                phi[mt][r] = (short)(pu >> 16);
-                plo[mt][r] = (short)f32_to_bf16(p - __uint_as_float(pu & 0xffff0000u));
-            }
-        lsum += __shfl_xor(lsum, 16, WAVE);
-        lsum += __shfl_xor(lsum, 32, WAVE);
-        l = l * corr + lsum;
-        m = mnew;
+            for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float p = __builtin_amdgcn_exp2f(sc[u][mt][r] - msub);
+                    lsum += p;
+                    // hi = p truncated to bf16 (exact remainder), lo = remainder rounded
+                    const uint32_t pu = __float_as_uint(p);
+                    phi[u][mt][r] = (short)(pu >> 16);
+                    plo[u][mt][r] = (short)f32_to_bf16(p - __uint_as_float(pu & 0xffff0000u));
+                }
+            lsum += __shfl_xor(lsum, 16, WAVE);
+            lsum += __shfl_xor(lsum, 32, WAVE);
+            l[u] = l[u] * corr[u] + lsum;
+            m[u] = mnew;
+        }
 #pragma unroll
         for (int dt = 0; dt < MAXDV; ++dt) {
             if (16 * dt < Dv) {
-                o[dt] *= corr;
+#pragma unroll
+                for (int u = 0; u < NT; ++u) o[u][dt] *= corr[u];
                 const bf16s* vr = Vt + (16 * dt + lc) * vst + 4 * lg;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb) {
                     const s4_t a0 = *reinterpret_cast<const s4_t*>(vr + 32 * kb);
                     const s4_t a1 = *reinterpret_cast<const s4_t*>(vr + 32 * kb + 16);
                     const s8_t a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
-                    const s8_t bh = __builtin_shufflevector(phi[2 * kb], phi[2 * kb + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                    const s8_t bl = __builtin_shufflevector(plo[2 * kb], plo[2 * kb + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bh, o[dt], 0, 0, 0);
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bl, o[dt], 0, 0, 0);
+#pragma unroll
+                    for (int u = 0; u < NT; ++u) {
+                        const s8_t bh = __builtin_shufflevector(phi[u][2 * kb], phi[u][2 * kb + 1],
+                                                                0, 1, 2, 3, 4, 5, 6, 7);
+                        const s8_t bl = __builtin_shufflevector(plo[u][2 * kb], plo[u][2 * kb + 1],
+                                                                0, 1, 2, 3, 4, 5, 6, 7);
+                        o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bh, o[u][dt], 0, 0, 0);
+                        o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bl, o[u][dt], 0, 0, 0);
+                    }
                 }
             }
         }
     }
-    if (lc >= ntok) return;
-    const int tok = lo + t0 + lc;
-    if (nsplit == 1) {
-        const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) / l;
-        bf16s* orow = out + ((int64_t)tok * H + h) * Dv + 4 * lg;
 #pragma unroll
-        for (int dt = 0; dt < MAXDV; ++dt)
-            if (16 * dt < Dv) {
-                uint2 w;
-                w.x = pack_bf16x2(o[dt][0] * gt, o[dt][1] * gt);
-                w.y = pack_bf16x2(o[dt][2] * gt, o[dt][3] * gt);
-                *reinterpret_cast<uint2*>(orow + 16 * dt) = w;
+    for (int u = 0; u < NT; ++u) {
+        if (lc >= ntok[u]) continue;
+        const int tok = lo + t0 + 16 * u + lc;
+        if (nsplit == 1) {
+            const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) / l[u];
+            bf16s* orow = out + ((int64_t)tok * H + h) * Dv + 4 * lg;
+#pragma unroll
+            for (int dt = 0; dt < MAXDV; ++dt)
+                if (16 * dt < Dv) {
+                    uint2 w;
+                    w.x = pack_bf16x2(o[u][dt][0] * gt, o[u][dt][1] * gt);
+                    w.y = pack_bf16x2(o[u][dt][2] * gt, o[u][dt][3] * gt);
+                    *reinterpret_cast<uint2*>(orow + 16 * dt) = w;
+                }
+        } else {
+            const int64_t pr = ((int64_t)tok * H + h) * nsplit + split;
+#pragma unroll
+            for (int dt = 0; dt < MAXDV; ++dt)
+                if (16 * dt < Dv)
+                    *reinterpret_cast<f4_t*>(part_o + pr * Dv + 16 * dt + 4 * lg) = o[u][dt];
+            if (lg == 0) {
+                part_ml[pr * 2] = m[u] * 0.6931471805599453f;   // back to the natural-log domain
+                part_ml[pr * 2 + 1] = l[u];
             }
-    } else {
-        const int64_t pr = ((int64_t)tok * H + h) * nsplit + split;
-#pragma unroll
-        for (int dt = 0; dt < MAXDV; ++dt)
-            if (16 * dt < Dv)
-                *reinterpret_cast<f4_t*>(part_o + pr * Dv + 16 * dt + 4 * lg) = o[dt];
-        if (lg == 0) {
-            part_ml[pr * 2] = m * 0.6931471805599453f;   // back to the natural-log domain
-            part_ml[pr * 2 + 1] = l;
         }
     }
 }
@@ -1301,12 +1332,21 @@ static int attn_path(int H, int G, int D, int Dv, int dt) {
 }
 static int attn_hb(int R) { return R % 4 == 0 ? 4 : (R % 2 == 0 ? 2 : 1); }
 
-extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int* TQ, int* KT,
-                                     int* kstride, int* lds_bytes) {
+// token sub-tiles per wave of the matrix-core kernel. Two sub-tiles halve
+// the LDS fragment reads and the staging per query row, but at 128-wide
+// heads they need ~300 registers per lane (one wave per SIMD) and measured
+// no faster than one sub-tile at three waves per SIMD; one is used.
+static int attn_nt(int D, int Dv, int max_chunk) {
+    (void)D; (void)Dv; (void)max_chunk;
+    return 1;
+}
+
+extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int max_chunk, int* TQ,
+                                     int* KT, int* kstride, int* lds_bytes) {
     if (G < 1 || H % G != 0 || Dv > 64 * ATT_MAXV) return -100;
     const int R = H / G;
     if (attn_path(H, G, D, Dv, dt)) {
-        *TQ = 16 * (4 / attn_hb(R));
+        *TQ = 16 * (4 / attn_hb(R)) * attn_nt(D, Dv, max_chunk);
         *KT = MF_KT;
         *kstride = D + MF_KPAD;
         *lds_bytes = (MF_KT * (D + MF_KPAD) + Dv * (MF_KT + 4)) * 2;
@@ -1328,7 +1368,7 @@ extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int* T
     return -103;
 }
 
-template <int MAXD, int MAXDV, bool QK32>
+template <int MAXD, int MAXDV, bool QK32, int NT>
 static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void* q, const void* gate,
                              int64_t gs, const void* k_cache, const void* v_cache, void* out,
                              void* part_o, void* part_ml, const void* cu, const void* past,
@@ -1336,9 +1376,9 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                              const void* slopes, int B, int H, int G, int D, int Dv, int HB,
                              float scale, int nsplit) {
     if (lds_bytes > 48 * 1024)
-        (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV, QK32>,
+        (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV, QK32, NT>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    hipLaunchKernelGGL((attn_bias_mfma_kernel<MAXD, MAXDV, QK32>), grid, dim3(256), lds_bytes, s,
+    hipLaunchKernelGGL((attn_bias_mfma_kernel<MAXD, MAXDV, QK32, NT>), grid, dim3(256), lds_bytes, s,
                        (const bf16s*)q, (const bf16s*)gate, gs, (const bf16s*)k_cache,
                        (const bf16s*)v_cache, (bf16s*)out, (float*)part_o, (float*)part_ml,
                        (const int*)cu, (const int*)past, (const int*)block_table, max_blocks,
@@ -1351,26 +1391,23 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
                                   void* part_o, void* part_ml, const void* cu, const void* past,
                                   const void* block_table, int max_blocks, int block_size,
                                   const void* slopes, int T, int B, int ntiles, int H, int G,
-                                  int D, int Dv, float scale, int nsplit, int dt) {
+                                  int D, int Dv, float scale, int nsplit, int dt, int max_chunk) {
     if (T <= 0 || ntiles <= 0) return 0;
     int TQ, KT, ks, lds_bytes;
-    int rc = oa_attn_bias_geometry(H, G, D, Dv, dt, &TQ, &KT, &ks, &lds_bytes);
+    int rc = oa_attn_bias_geometry(H, G, D, Dv, dt, max_chunk, &TQ, &KT, &ks, &lds_bytes);
     if (rc) return rc;
     if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return -104;
     hipStream_t s = (hipStream_t)stream;
     if (attn_path(H, G, D, Dv, dt)) {
         const int R = H / G, HB = attn_hb(R);
         dim3 grid(ntiles, G * (R / HB), nsplit);
-#define MF(A, Bv)                                                                                   \
-    do {                                                                                            \
-        if (D % 32 == 0)                                                                            \
-            launch_attn_mfma<A, Bv, true>(s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out,   \
-                                          part_o, part_ml, cu, past, block_table, max_blocks,       \
-                                          block_size, slopes, B, H, G, D, Dv, HB, scale, nsplit);   \
-        else                                                                                        \
-            launch_attn_mfma<A, Bv, false>(s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out,  \
-                                           part_o, part_ml, cu, past, block_table, max_blocks,      \
-                                           block_size, slopes, B, H, G, D, Dv, HB, scale, nsplit);  \
+#define MF_ARGS                                                                                   \
+    s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out, part_o, part_ml, cu, past, block_table, \
+        max_blocks, block_size, slopes, B, H, G, D, Dv, HB, scale, nsplit
+#define MF(A, Bv)                                                               \
+    do {                                                                        \
+        if (D % 32 == 0) launch_attn_mfma<A, Bv, true, 1>(MF_ARGS);             \
+        else launch_attn_mfma<A, Bv, false, 1>(MF_ARGS);                        \
     } while (0)
         const int a = D <= 64 ? 4 : (D <= 128 ? 8 : 16), bv = Dv <= 64 ? 4 : (Dv <= 128 ? 8 : 16);
         if (a == 4 && bv == 4) MF(4, 4);
@@ -1383,6 +1420,7 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
         else if (bv == 8) MF(16, 8);
         else MF(16, 16);
 #undef MF
+#undef MF_ARGS
         HIP_CHECK_LAUNCH();
     } else {
         dim3 grid(ntiles, G, nsplit), blk(256);

@@ -121,9 +121,9 @@ def _declare_mixers(lib: ctypes.CDLL) -> None:
         "oa_causal_conv_seq": [p, p, i64, i, p, p, p, i64, p, p, p, p, i, i, i, i, i, i, i, i],
         "oa_group_rmsnorm": [p, p, i64, i, p, p, p, i, i, i, f, i],
         "oa_attn_prepare": [p, p, i64, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i],
-        "oa_attn_bias_geometry": [i, i, i, i, i, ip, ip, ip, ip],
+        "oa_attn_bias_geometry": [i, i, i, i, i, i, ip, ip, ip, ip],
         "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p,
-                               i, i, i, i, i, i, i, f, i, i],
+                               i, i, i, i, i, i, i, f, i, i, i],
         "oa_delta_rule_fused": [p, p, i64, p, i64, p, i64, p, i64, p, i64, p, p, p, p, i64,
                                 p, p, p, p, p, p, i, i, i, i, i, i, f, i, i],
         "oa_softcap": [p, p, p, i64, f, i],

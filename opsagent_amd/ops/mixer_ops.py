@@ -184,13 +184,15 @@ def attn_qkv_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm_w: 
 _GEOM = {}
 
 
-def attn_geometry(H: int, G: int, D: int, Dv: int, dt: int) -> Tuple[int, int]:
-    """(query tokens per tile, keys per staged tile) of the attention kernel."""
-    key = (H, G, D, Dv, dt)
+def attn_geometry(H: int, G: int, D: int, Dv: int, dt: int, max_chunk: int) -> Tuple[int, int]:
+    """(query tokens per tile, keys per staged tile) of the attention kernel
+    for steps whose longest portion is max_chunk tokens."""
+    key = (H, G, D, Dv, dt, max_chunk >= 32)
     if key not in _GEOM:
         lib, hip = _lib()
         vals = [ctypes.c_int() for _ in range(4)]
-        rc = lib.oa_attn_bias_geometry(H, G, D, Dv, dt, *[ctypes.byref(v) for v in vals])
+        rc = lib.oa_attn_bias_geometry(H, G, D, Dv, dt, max_chunk,
+                                       *[ctypes.byref(v) for v in vals])
         hip.check(rc, "oa_attn_bias_geometry")
         _GEOM[key] = (vals[0].value, vals[1].value)
     return _GEOM[key]
@@ -209,7 +211,7 @@ def attention_biased_paged(q: torch.Tensor, gate_logits: torch.Tensor, k_cache: 
                                                 sb.past, sb.block_table, scale, slopes)
     lib, hip = _lib()
     dt = _dt(q)
-    TQ, KT = attn_geometry(H, G, D, Dv, dt)
+    TQ, KT = attn_geometry(H, G, D, Dv, dt, sb.max_chunk)
     ntiles = sum((sb.cu[b + 1] - sb.cu[b] + TQ - 1) // TQ for b in range(sb.num_seqs))
     # few tiles and long contexts: split the keys over blocks to fill the chip
     nkt = max(1, (sb.max_total + KT - 1) // KT)
@@ -229,7 +231,7 @@ def attention_biased_paged(q: torch.Tensor, gate_logits: torch.Tensor, k_cache: 
         part_ml.data_ptr() if part_ml is not None else None,
         sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.block_table.data_ptr(),
         sb.block_table.shape[1], bs, slopes.data_ptr(), T, sb.num_seqs, ntiles, H, G, D, Dv,
-        float(scale), nsplit, dt)
+        float(scale), nsplit, dt, sb.max_chunk)
     hip.check(rc, "oa_attn_bias_paged")
     return out
 

@@ -47,3 +47,15 @@ def test_grammar_library_exports():
               "oa_grammar_completion", "oa_grammar_is_complete",
               "oa_grammar_reset", "oa_vocab_create", "oa_vocab_destroy"]:
         assert hasattr(lib, s), f"missing {s}"
+
+
+MIXERS_LIB = LIB.replace("libopsagent_kernels", "libopsagent_mixers")
+
+
+@pytest.mark.skipif(not os.path.exists(MIXERS_LIB), reason="mixers .so not built")
+def test_mixers_library_exports():
+    lib = ctypes.CDLL(MIXERS_LIB)
+    for s in ["oa_causal_conv_seq", "oa_group_rmsnorm", "oa_attn_prepare",
+              "oa_attn_bias_geometry", "oa_attn_bias_paged", "oa_delta_rule_fused",
+              "oa_softcap", "oa_silu_mul_rows", "oa_embed_rows"]:
+        assert hasattr(lib, s), f"missing {s}"
