@@ -146,6 +146,9 @@ class LLMEngine:
             if not self.hybrid:
                 raise ValueError("float32 serving is implemented for hybrid models only")
             self.dtype = torch.float32
+            # true 32-bit library GEMMs: no reduced-precision matrix mode
+            torch.backends.cuda.matmul.allow_tf32 = False
+            torch.set_float32_matmul_precision("highest")
         else:
             self.dtype = torch.float16
         self.max_batch = int(cfg.get("max_batch_size", 64))

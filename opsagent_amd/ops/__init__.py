@@ -85,6 +85,11 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         and x.shape[-1] % 8 == 0
         and w.stride(1) == 1
         and x.is_contiguous()
+        # the kernels read 16 bytes at a time: a column slice of a wider
+        # buffer may start anywhere
+        and x.data_ptr() % 16 == 0
+        and w.data_ptr() % 16 == 0
+        and w.stride(0) % 8 == 0
     ):
         from opsagent_amd.ops import hip_lib
 

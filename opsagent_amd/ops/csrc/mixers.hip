@@ -459,11 +459,15 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
     const int* __restrict__ cu, const int* __restrict__ past,
     const int* __restrict__ block_table, int max_blocks, int block_size,
     const float* __restrict__ slopes, int B, int H, int G, int D, int Dv, int TQ,
-    int KT, int kstride, float scale, int nsplit) {
+    int KT, int kstride, float scale, int nsplit, int RB) {
     extern __shared__ float lds[];
-    const int R = H / G;
+    // a block takes up to RB of the H/G query heads of one kv head
+    const int hgroups = (H / G + RB - 1) / RB;
+    const int g = blockIdx.y / hgroups;
+    const int h0 = g * (H / G) + (blockIdx.y % hgroups) * RB;
+    const int R = min(RB, (g + 1) * (H / G) - h0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int g = blockIdx.y, split = blockIdx.z;
+    const int split = blockIdx.z;
     // locate this block's tile: walk the sequences
     int tile = blockIdx.x, b = 0, lo = 0, n = 0;
     for (; b < B; ++b) {
@@ -481,14 +485,14 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
     const int last_pos = p0 + nq_tok - 1;
     const int* bt = block_table + (int64_t)b * max_blocks;
 
-    float* Qs = lds;                                // [TQ*R][D]
-    float* Ps = Qs + (size_t)TQ * R * D;            // [4][KT]
+    float* Qs = lds;                                // [TQ*RB][D]
+    float* Ps = Qs + (size_t)TQ * RB * D;           // [4][KT]
     TC* Ks = (TC*)(Ps + 4 * KT);                    // [KT][kstride]
     TC* Vs = Ks + (size_t)KT * kstride;             // [KT][Dv]
 
     for (int i = threadIdx.x; i < rows * D; i += blockDim.x) {
         const int r = i / D, d = i % D;
-        const int tok = lo + t0 + r / R, h = g * R + r % R;
+        const int tok = lo + t0 + r / R, h = h0 + r % R;
         Qs[i] = ldf(q, ((int64_t)tok * H + h) * D + d) * scale;
     }
     float m[ATT_MAXR], l[ATT_MAXR], acc[ATT_MAXR][ATT_MAXV];
@@ -523,7 +527,7 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
             if (r >= rows) break;
             const int pos = p0 + r / R;
             if (k0 > pos) continue;
-            const float slope = slopes[g * R + r % R];
+            const float slope = slopes[h0 + r % R];
             float s = -INFINITY;
             if (lane < nk && k0 + lane <= pos) {
                 const float* qr = Qs + r * D;
@@ -558,7 +562,7 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
     for (int ri = 0; ri < ATT_MAXR; ++ri) {
         const int r = wave + 4 * ri;
         if (r >= rows) break;
-        const int tok = lo + t0 + r / R, h = g * R + r % R;
+        const int tok = lo + t0 + r / R, h = h0 + r % R;
         if (nsplit == 1) {
             const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h));
             const float inv = gt / l[ri];
@@ -1352,14 +1356,14 @@ extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int ma
         *lds_bytes = (MF_KT * (D + MF_KPAD) + Dv * (MF_KT + 4)) * 2;
         return 0;
     }
-    if (R > 4 * ATT_MAXR) return -102;
-    int tq = std::max(1, (4 * ATT_MAXR) / R);
+    const int rb = std::min(R, 4 * ATT_MAXR);        // query heads per block
+    int tq = std::max(1, (4 * ATT_MAXR) / rb);
     const int esz = dt == 1 ? 4 : 2;
     int ks = D;
     if (dt == 1) ks = (D % 2 == 0) ? D + 1 : D;
     else ks = ((D / 2) % 2 == 0) ? D + 2 : D + (D % 2);
     for (int kt = 64; kt >= 8; kt >>= 1) {
-        size_t bytes = ((size_t)tq * R * D + 4 * kt) * 4 + ((size_t)kt * ks + (size_t)kt * Dv) * esz;
+        size_t bytes = ((size_t)tq * rb * D + 4 * kt) * 4 + ((size_t)kt * ks + (size_t)kt * Dv) * esz;
         if (bytes <= 64 * 1024) {
             *TQ = tq; *KT = kt; *kstride = ks; *lds_bytes = (int)bytes;
             return 0;
@@ -1423,12 +1427,13 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
 #undef MF_ARGS
         HIP_CHECK_LAUNCH();
     } else {
-        dim3 grid(ntiles, G, nsplit), blk(256);
+        const int rb = std::min(H / G, 4 * ATT_MAXR);
+        dim3 grid(ntiles, G * CEIL_DIV(H / G, rb), nsplit), blk(256);
 #define AT_ARGS(TC)                                                                      \
     (const TC*)q, (const TC*)gate, gs, (const TC*)k_cache, (const TC*)v_cache, (TC*)out,  \
         (float*)part_o, (float*)part_ml, (const int*)cu, (const int*)past,                \
         (const int*)block_table, max_blocks, block_size, (const float*)slopes, B, H, G, D, \
-        Dv, TQ, KT, ks, scale, nsplit
+        Dv, TQ, KT, ks, scale, nsplit, rb
         if (dt == 1)
             hipLaunchKernelGGL((attn_bias_paged_kernel<float>), grid, blk, lds_bytes, s, AT_ARGS(float));
         else

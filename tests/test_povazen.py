@@ -198,7 +198,7 @@ def _single_layer(kind, dtype, device, seed=0, **kw):
 # (heads, kv_heads, dim, vdim): ratios 1..4 and sizes that do and do not
 # divide by 16 (matrix-core and VALU kernels on the GPU)
 ATT_GEOMS = [(6, 2, 24, 40), (6, 2, 32, 48), (8, 2, 16, 80), (4, 2, 64, 16), (2, 2, 160, 32),
-             (3, 1, 144, 144)]
+             (3, 1, 144, 144), (20, 1, 8, 8)]
 
 
 @pytest.mark.parametrize("mode", MODES)
@@ -464,7 +464,7 @@ def test_long_decode(mode):
 
 
 @pytest.mark.parametrize("mode", MODES)
-@pytest.mark.parametrize("variant", ["equal-sizes", "ones", "wide-head"])
+@pytest.mark.parametrize("variant", ["equal-sizes", "ones", "wide-head", "one-tap"])
 def test_other_sizes(mode, variant):
     """Sizes that another checkpoint may choose: key size == value size,
     kv_heads == heads; single head, single group, two taps; 160-wide keys."""
@@ -476,6 +476,8 @@ def test_other_sizes(mode, variant):
     elif variant == "ones":
         cfg = make_cfg(pattern="dA", heads=1, kv_heads=1, dim=8, vdim=8, d_heads=1, d_kv=1,
                        d_dim=8, d_vdim=8, width=16, groups=1, taps=2, conv=2, ff=24, vocab=33)
+    elif variant == "one-tap":
+        cfg = make_cfg(pattern="Da", taps=1, conv=1)
     else:
         cfg = make_cfg(pattern="AD", heads=2, kv_heads=1, dim=160, vdim=72, d_heads=2, d_kv=1,
                        d_dim=136, d_vdim=72, width=40, groups=5, taps=4, conv=5)
