@@ -128,7 +128,7 @@ def main() -> None:
     from opsagent_amd.parallel import state as pstate
 
     have_gpu = torch.cuda.is_available()
-    # real-tokenizer default (VERDICT r1 #5): the committed 32k byte-level
+    # real-tokenizer default: the committed 32k byte-level
     # BPE; --tokenizer byte reverts to the raw byte vocabulary
     tok_path = None
     if args.tokenizer == "auto":
@@ -190,7 +190,7 @@ def main() -> None:
     total_prefill_tokens = 0
 
     if world > 1 and rank != 0:
-        # Followers never see the request stream (VERDICT r1 #1): rank 0
+        # Followers never see the request stream: rank 0
         # broadcasts tokenized admissions inside engine.step(); marks from
         # bcast_mark() delimit the warmup and timed regions here.
         reason = eng.follower_loop()            # ... until end-of-warmup mark

@@ -144,7 +144,7 @@ class ChatCompletionAPI:
         # Holdback covers the worst case trim: the engine trims WHOLE tokens
         # when a stop matches, so up to (max stop bytes - 1) + (max token
         # bytes - 1) already-queued bytes can disappear from the final output
-        # (ADVICE r1). Byte-level vocab: max_token_bytes == 1 → plain stop len.
+        # Byte-level vocab: max_token_bytes == 1 → plain stop len.
         holdback = max((len(s.encode("utf-8")) for s in stops), default=0)
         if holdback:
             holdback += max(0, getattr(tok, "max_token_bytes", 1) - 1)

@@ -357,7 +357,6 @@ def moe_grouped_mlp(
       * expert-major (P > OPSAGENT_MOE_EMAJ_MIN_P, needs num_experts): one
         block column per EXPERT; weights stream once per GROUP of 8 matched
         pairs, cutting the weight traffic up to 8x at big decode batches
-        (VERDICT r1 #7 — keeps large-batch MoE graph-capturable)
     """
     assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous()
     # stride-0 expand views have a data_ptr that covers ONE element — the

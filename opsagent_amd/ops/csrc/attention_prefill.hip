@@ -2,7 +2,7 @@
 // "Prefill attention kernel (HIP, bf16 MFMA, LDS-staged KV tiles, gfx950
 // tiling)".
 //
-// v2 structure (close the pipelining gap):
+// v2 structure:
 //   * workgroup = 512 threads = 8 waves; wave owns RB x 16 q-rows
 //     (RB=2 -> 256-row q-tile; RB=1 -> 128-row tile used when the grid
 //     would underfill the 256 CUs at small Sq)

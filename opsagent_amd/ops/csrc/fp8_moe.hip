@@ -583,7 +583,7 @@ extern "C" int oa_gemv_gateup_fp8(void* stream, const void* x, const void* w8,
 // ---- fp8 MFMA tile GEMM (prefill path) -------------------------------------
 // C[M, N] = (A8[M, K] @ B8[N, K]^T) * a_scale[m] * b_scale[n], bf16 out.
 //
-// v2 (VERDICT r1 #3 — pipeline the fp8 GEMM): 128x128 tile, 4 waves (2x2 of
+// v2: 128x128 tile, 4 waves (2x2 of
 // 64x64), K-step 128 fp8 bytes (2x the old unroll -> half the barriers), A/B
 // staged by 16-B global_load_lds into a DOUBLE-BUFFERED ring (the guide's
 // step-3 '+67%' lever over register staging, and its verified 2-buffer

@@ -91,7 +91,7 @@ def create_app(cfg: Optional[Config] = None) -> FastAPI:
     jwt_expire = int(cfg.get("jwt.expire", 24))
     started_at = time.time()
 
-    # Loud warning for shipped defaults (ADVICE r1): admin/novastar and the
+    # Loud warning for shipped defaults: admin/novastar and the
     # well-known jwt key are reference-compatible but must be overridden in
     # any real deployment (deploy/ manifests inject both via Secrets).
     if str(cfg.get("auth.password", DEFAULT_PASSWORD)) == DEFAULT_PASSWORD:
@@ -338,7 +338,7 @@ def create_app(cfg: Optional[Config] = None) -> FastAPI:
 
     # -- OpenAI-compatible endpoints over the local engine -----------------
     #
-    # Gated (ADVICE r1, medium): unauthenticated /v1 would let any network
+    # Gated: unauthenticated /v1 would let any network
     # peer drive the GPU engine. Accepts a valid JWT bearer OR an X-API-Key
     # matching engine.api_key; `engine.open_api: true` opts out explicitly
     # (e.g. for a localhost-only sidecar deployment).

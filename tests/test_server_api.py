@@ -138,7 +138,7 @@ def test_jwt_tamper_rejected():
 
 def test_v1_models_listing(client_and_llm):
     client, _ = client_and_llm
-    # /v1 is gated (ADVICE r1): no credentials -> 401
+    # /v1 is gated: no credentials -> 401
     r = client.get("/v1/models")
     assert r.status_code == 401
     token = login(client)

@@ -109,7 +109,7 @@ def test_bpe_forced_peek_nonadvancing(bpe_path):
 
 
 def test_bpe_jump_ahead_token_aligned(bpe_path):
-    """BPE jump-ahead (VERDICT r1 #5): the engine appends whole BPE tokens
+    """BPE jump-ahead: the engine appends whole BPE tokens
     for forced template literals without model passes; output still parses
     as the exact ToolPrompt schema and forced-run catch-ups were used."""
     from opsagent_amd.engine.engine import LLMEngine, SamplingParams

@@ -1,7 +1,7 @@
 """Tensor-parallel tests over gloo (CPU, world_size 2 and 4).
 
 SURVEY.md §4 (e): TP sharding equivalence TP=k vs TP=1 on the same random
-weights. Uses the PRODUCTION request topology (VERDICT r1 #1): rank 0 owns
+weights. Uses the PRODUCTION request topology: rank 0 owns
 the request stream (generate / EngineLoop / HTTP server); follower ranks
 mirror its steps via the engine's per-step admission broadcast
 (engine.follower_loop). Because weights are drawn full-size from a fixed
@@ -127,7 +127,7 @@ def test_shard_helper():
 
 # ---------------------------------------------------------------------------
 # tp=8 shard math at the 70B head geometry (Hq=64, Hk=8 → hk_local=1, G=8)
-# — model construction per rank, no process group needed (VERDICT r1 weak #5)
+# — model construction per rank, no process group needed
 # ---------------------------------------------------------------------------
 def test_tp8_shard_shapes_70b_geometry():
     import dataclasses
@@ -247,7 +247,7 @@ def test_tp2_features_match_tp1():
 
 # ---------------------------------------------------------------------------
 # HTTP /api/execute round-trip on a world=2 engine: the server runs ONLY on
-# rank 0; rank 1 is a pure follower (VERDICT r1 #1 "Done" criterion)
+# rank 0; rank 1 is a pure follower
 # ---------------------------------------------------------------------------
 def _run_http_worker(rank: int, world: int, port: int, q):
     dist = _init_dist(rank, world, port)
