@@ -686,6 +686,11 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
             }
         }
     }
+    float kbias[4][4];                       // slope * (16*mt + r), exp2 domain
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) kbias[mt][r] = slope * (float)(16 * mt + r);
     f4_t o[NT][MAXDV];
     float m[NT], l[NT];
 #pragma unroll
@@ -698,48 +703,61 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
 
     const int nkt = block_last / MF_KT + 1;
     const int dch = D / 8, vch = Dv / 8;
-    // pages are a power of two: shifts, not divisions, in the staging loops
+    // pages are a power of two: shifts, not divisions
     const int bsh = 31 - __clz(block_size), bmask = block_size - 1;
-    const int kj0 = threadIdx.x / dch, kc0 = threadIdx.x % dch;
-    const int kjs = 256 / dch, kcs = 256 % dch;
-    for (int kt = split; kt < nkt; kt += nsplit) {
+    // Staging map: a thread owns ONE key per tile for K (key tid/4, every 4th
+    // 16-byte piece of its row) and one for V (key tid%64, every 4th piece),
+    // so a tile costs it two page lookups. The next tile's pieces are loaded
+    // into registers while the current tile is computed.
+    constexpr int KC = MAXD / 2, VC = MAXDV / 2;
+    const int kj = threadIdx.x >> 2, kc0 = threadIdx.x & 3;
+    const int vj = threadIdx.x & 63, vc0 = threadIdx.x >> 6;
+    uint4 kreg[KC], vreg[VC];
+    auto fetch = [&](int kt) {
         const int k0 = kt * MF_KT;
         const int nk = min(MF_KT, block_last + 1 - k0);
-        __syncthreads();
-        {   // K rows: (key j, 8-wide piece c) walks forward by 256 pieces per step
-            int j = kj0, c = kc0;
-            for (int i = threadIdx.x; i < MF_KT * dch; i += 256) {
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (j < nk) {
-                    const int key = k0 + j;
-                    const int64_t slot = ((int64_t)bt[key >> bsh] << bsh) + (key & bmask);
-                    v = *reinterpret_cast<const uint4*>(k_cache + (slot * G + g) * D + 8 * c);
-                }
-                *reinterpret_cast<uint4*>(Ks + j * kst + 8 * c) = v;
-                j += kjs;
-                c += kcs;
-                if (c >= dch) {
-                    c -= dch;
-                    ++j;
-                }
-            }
-        }
-        for (int i = threadIdx.x; i < MF_KT * vch; i += 256) {
-            const int j = i % MF_KT, c = i / MF_KT;   // lanes along keys: adjacent LDS columns
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (j < nk) {
-                const int key = k0 + j;
-                const int64_t slot = ((int64_t)bt[key >> bsh] << bsh) + (key & bmask);
-                v = *reinterpret_cast<const uint4*>(v_cache + (slot * G + g) * Dv + 8 * c);
-            }
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const int keyk = k0 + kj, keyv = k0 + vj;
+        const bool okk = kj < nk, okv = vj < nk;
+        const int64_t sk_ = okk ? ((int64_t)bt[keyk >> bsh] << bsh) + (keyk & bmask) : 0;
+        const int64_t sv_ = okv ? ((int64_t)bt[keyv >> bsh] << bsh) + (keyv & bmask) : 0;
+        const bf16s* kp = k_cache + (sk_ * G + g) * D;
+        const bf16s* vp = v_cache + (sv_ * G + g) * Dv;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                Vt[(8 * c + 2 * e) * vst + j] = (bf16s)(w[e] & 0xffffu);
-                Vt[(8 * c + 2 * e + 1) * vst + j] = (bf16s)(w[e] >> 16);
+        for (int u = 0; u < KC; ++u) {
+            const int c = kc0 + 4 * u;
+            kreg[u] = (okk && c < dch) ? *reinterpret_cast<const uint4*>(kp + 8 * c)
+                                       : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < VC; ++u) {
+            const int c = vc0 + 4 * u;
+            vreg[u] = (okv && c < vch) ? *reinterpret_cast<const uint4*>(vp + 8 * c)
+                                       : make_uint4(0, 0, 0, 0);
+        }
+    };
+    if (split < nkt) fetch(split);
+    for (int kt = split; kt < nkt; kt += nsplit) {
+        const int k0 = kt * MF_KT;
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < KC; ++u) {
+            const int c = kc0 + 4 * u;
+            if (c < dch) *reinterpret_cast<uint4*>(Ks + kj * kst + 8 * c) = kreg[u];
+        }
+#pragma unroll
+        for (int u = 0; u < VC; ++u) {
+            const int c = vc0 + 4 * u;
+            if (c < vch) {
+                const uint32_t w[4] = {vreg[u].x, vreg[u].y, vreg[u].z, vreg[u].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    Vt[(8 * c + 2 * e) * vst + vj] = (bf16s)(w[e] & 0xffffu);
+                    Vt[(8 * c + 2 * e + 1) * vst + vj] = (bf16s)(w[e] >> 16);
+                }
             }
         }
         __syncthreads();
+        if (kt + nsplit < nkt) fetch(kt + nsplit);
         if (wave_ntok <= 0 || k0 > wave_last) continue;
         // S^T tiles: keys k0 + 16*mt + 4*lg + r, token lc of sub-tile u
         f4_t sc[NT][4];
@@ -774,14 +792,19 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         float corr[NT];
 #pragma unroll
         for (int u = 0; u < NT; ++u) {
+            // score = s*scale2 - slope*(pos - key), key = k0 + 16*mt + 4*lg + r:
+            // the key part is a per-lane constant table, the rest one value
+            // per tile, so an element costs one add and one fma
+            const float base = slope * (float)(pos[u] - k0 - 4 * lg);
             float mloc = -INFINITY;
+            // only tiles that reach past some token of the wave need the mask
+            const bool diag = k0 + MF_KT - 1 > pb + t0 + 16 * u;
 #pragma unroll
             for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const int key = k0 + 16 * mt + 4 * lg + r;
-                    float v = sc[u][mt][r] * scale2 - slope * (float)(pos[u] - key);
-                    v = (key <= pos[u]) ? v : -INFINITY;
+                    float v = fmaf(sc[u][mt][r], scale2, kbias[mt][r] - base);
+                    if (diag) v = (k0 + 16 * mt + 4 * lg + r <= pos[u]) ? v : -INFINITY;
                     sc[u][mt][r] = v;
                     mloc = fmaxf(mloc, v);
                 }
@@ -799,10 +822,12 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
                 for (int r = 0; r < 4; ++r) {
                     const float p = __builtin_amdgcn_exp2f(sc[u][mt][r] - msub);
                     lsum += p;
-                    // hi = p truncated to bf16 (exact remainder), lo = remainder rounded
+                    // p = hi + lo + (less than 2^-16 p): both halves by
+                    // truncation, so the first remainder is exact
                     const uint32_t pu = __float_as_uint(p);
                     phi[u][mt][r] = (short)(pu >> 16);
-                    plo[u][mt][r] = (short)f32_to_bf16(p - __uint_as_float(pu & 0xffff0000u));
+                    const float rem = p - __uint_as_float(pu & 0xffff0000u);
+                    plo[u][mt][r] = (short)(__float_as_uint(rem) >> 16);
                 }
             lsum += __shfl_xor(lsum, 16, WAVE);
             lsum += __shfl_xor(lsum, 32, WAVE);
@@ -1001,23 +1026,36 @@ __global__ void delta_fused_kernel(
     for (int c0 = 0; c0 < n; c0 += TCK) {
         const int nc = min(TCK, n - c0);
         const int tb = lo + c0;
-        for (int i = tid; i < nc * DP; i += nth) {
-            const int tt = i / DP, r = i % DP;
-            const int64_t t = tb + tt;
-            float qv = 0.0f, kv = 0.0f, gv = 0.0f;
-            if (r < D) {
-                qv = ldf(q, t * qs + kvh * D + r);
-                kv = ldf(k, t * ks + kvh * D + r);
-                const float z = ldf(a, t * as + h * D + r) + ldf(dt_bias, h * D + r);
-                gv = expf(-A * softplusf_(z));
+        // four pieces per thread and pass: all loads are issued before any
+        // of the softplus/exp chains, so their latencies overlap
+        for (int i0 = tid; i0 < nc * DP; i0 += 4 * nth) {
+            float qv[4], kv[4], zv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = i0 + u * nth;
+                const int tt = i / DP, r = i % DP;
+                const int64_t t = tb + tt;
+                qv[u] = kv[u] = zv[u] = 0.0f;
+                if (i < nc * DP && r < D) {
+                    qv[u] = ldf(q, t * qs + kvh * D + r);
+                    kv[u] = ldf(k, t * ks + kvh * D + r);
+                    zv[u] = ldf(a, t * as + h * D + r) + ldf(dt_bias, h * D + r);
+                }
             }
-            sq[i] = qv;
-            sk[i] = kv;
-            sg[i] = gv;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = i0 + u * nth;
+                if (i < nc * DP) {
+                    sq[i] = qv[u];
+                    sk[i] = kv[u];
+                    sg[i] = (i % DP < D) ? expf(-A * softplusf_(zv[u])) : 0.0f;
+                }
+            }
         }
-        for (int i = tid; i < nc * Dv; i += nth) {
-            const int tt = i / Dv, c = i % Dv;
-            sv[i] = ldf(v, (int64_t)(tb + tt) * vs + h * Dv + c);
+        // only this block's share of the value columns is read
+        for (int i = tid; i < nc * cpb; i += nth) {
+            const int tt = i / cpb, c = cb + i % cpb;
+            sv[tt * Dv + c] = ldf(v, (int64_t)(tb + tt) * vs + h * Dv + c);
         }
         for (int tt = tid; tt < nc; tt += nth)
             sb[tt] = sigmoidf_(ldf(bl, (int64_t)(tb + tt) * bs + h));
