@@ -300,7 +300,7 @@ class LLMEngine:
             self.kv = PagedKVCache(
                 self.spec.num_layers, 0, 0, self.block_size, num_blocks, self.device,
                 self.dtype, layer_shapes=self.model.kv_layer_shapes(),
-                prefix_caching=False, v_transposed=True,
+                prefix_caching=False,
             )
             self.state_pool = StateSlotPool(
                 int(cfg.get("state_slots", self.max_batch)),

@@ -38,17 +38,13 @@ class PagedKVCache:
         dtype: torch.dtype = torch.bfloat16,
         layer_shapes: Optional[Sequence[Optional[Tuple[int, int, int]]]] = None,
         prefix_caching: bool = True,
-        v_transposed: bool = False,
     ):
         """layer_shapes (optional) gives each layer's own (kv_heads, key dim,
         value dim), or None for a layer that keeps no keys and values (a
         recurrent mixer); without it every layer is [kv_heads, head_dim] for
         both. prefix_caching=False turns block publishing and reuse off: a
         model that also carries recurrent state cannot restart from cached
-        keys alone. v_transposed=True stores values page-wise transposed,
-        [blocks, kv_heads, value dim, block_size]: a page's keys are contiguous
-        per value channel, which is the layout the matrix-core attention kernel
-        stages (V^T tiles) without transposing."""
+        keys alone."""
         assert block_size & (block_size - 1) == 0, "block_size must be a power of 2"
         self.block_size = block_size
         self.num_blocks = num_blocks
@@ -63,10 +59,7 @@ class PagedKVCache:
                 continue
             hk, kdim, vdim = shape
             k = torch.zeros(num_blocks, block_size, hk, kdim, dtype=dtype, device=device)
-            if v_transposed:
-                v = torch.zeros(num_blocks, hk, vdim, block_size, dtype=dtype, device=device)
-            else:
-                v = torch.zeros(num_blocks, block_size, hk, vdim, dtype=dtype, device=device)
+            v = torch.zeros(num_blocks, block_size, hk, vdim, dtype=dtype, device=device)
             self.layers.append((k, v))
         # allocator state
         self._free: collections.deque[int] = collections.deque(range(num_blocks))

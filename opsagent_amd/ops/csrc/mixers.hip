@@ -300,7 +300,7 @@ __global__ __launch_bounds__(256) void attn_prepare_kernel(
     const TC* __restrict__ qw, const TC* __restrict__ kw, TC* __restrict__ q_out,
     TC* __restrict__ k_cache, TC* __restrict__ v_cache,
     const int* __restrict__ slot_mapping, const int* __restrict__ cu, int B, int H,
-    int G, int D, int Dv, float eps, int block_size) {
+    int G, int D, int Dv, float eps) {
     __shared__ float red[8];
     const int t = blockIdx.x;
     if (t >= cu[B]) return;  // padding row of a fixed-size (captured) launch
@@ -346,11 +346,8 @@ __global__ __launch_bounds__(256) void attn_prepare_kernel(
         }
         sv = wave_reduce_sum(sv);
         const float rv = 1.0f / sqrtf(sv / (float)Dv + eps);
-        // values are cached page-wise transposed: [blocks, G, Dv, block_size]
-        const int64_t vb = ((slot / block_size) * G + g) * (int64_t)Dv;
-        const int vo = (int)(slot % block_size);
         for (int i = lane; i < Dv; i += 64)
-            stf(v_cache, (vb + i) * block_size + vo, val(off + i) * rv);
+            stf(v_cache, slot * (int64_t)(G * Dv) + g * Dv + i, val(off + i) * rv);
     }
 }
 
@@ -361,7 +358,7 @@ __global__ __launch_bounds__(256) void attn_prepare_vec_kernel(
     const TC* __restrict__ qw, const TC* __restrict__ kw, TC* __restrict__ q_out,
     TC* __restrict__ k_cache, TC* __restrict__ v_cache,
     const int* __restrict__ slot_mapping, const int* __restrict__ cu, int B, int H,
-    int G, int D, int Dv, float eps, int block_size) {
+    int G, int D, int Dv, float eps) {
     __shared__ float red[8];
     const int t = blockIdx.x;
     if (t >= cu[B]) return;
@@ -430,13 +427,11 @@ __global__ __launch_bounds__(256) void attn_prepare_vec_kernel(
         }
         sv = wave_reduce_sum(sv);
         const float rv = 1.0f / sqrtf(sv / (float)Dv + eps);
-        // values are cached page-wise transposed: [blocks, G, Dv, block_size]
-        const int64_t vb = ((slot / block_size) * G + g) * (int64_t)Dv;
-        const int vo = (int)(slot % block_size);
         for (int i = lane * 8; i < Dv; i += 64 * 8) {
             val8(off + i, x);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) stf(v_cache, (vb + i + e) * block_size + vo, x[e] * rv);
+            for (int e = 0; e < 8; ++e) x[e] *= rv;
+            st8(v_cache, slot * (int64_t)(G * Dv) + g * Dv + i, x);
         }
     }
 }
@@ -522,8 +517,8 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
         for (int i = threadIdx.x; i < nk * Dv; i += blockDim.x) {
             const int j = i / Dv, d = i % Dv;
             const int key = k0 + j;
-            Vs[j * Dv + d] = v_cache[(((int64_t)bt[key / block_size] * G + g) * Dv + d) * block_size +
-                                     key % block_size];
+            const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
+            Vs[j * Dv + d] = v_cache[(slot * G + g) * Dv + d];
         }
         __syncthreads();
 #pragma unroll
@@ -606,9 +601,7 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
 // Scores, the distance penalty, softmax statistics and weights are float32;
 // a weight enters the value product as a bf16 pair hi + lo (two MFMAs), so
 // it keeps 16 bits of mantissa.
-// LDS: K tile [64][D+8], V^T tile [Dv][64+8] (bf16); the value cache is
-// page-wise transposed ([blocks, G, Dv, block_size]), so V^T tiles are copied,
-// not transposed. Pages hold a multiple of 8 keys.
+// LDS: K tile [64][D+8], V tile transposed [Dv][64+4] (bf16).
 // Where the key size divides by 32 (QK32) and always for the value product,
 // the gfx950 form v_mfma_f32_16x16x32_bf16 is used: same i/j mapping, a lane
 // holds k = 8*(lane>>4)..+7. The value product feeds it the weights a lane
@@ -620,7 +613,6 @@ typedef short s8_t __attribute__((ext_vector_type(8)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 #define MF_KT 64
 #define MF_KPAD 8
-#define MF_VPAD 8
 
 template <int MAXD, int MAXDV, bool QK32, int NT>
 __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
@@ -636,8 +628,8 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     extern __shared__ float lds[];
     bf16s* Ks = (bf16s*)lds;                        // [64][D+8]
     const int kst = D + MF_KPAD;
-    bf16s* Vt = Ks + (size_t)MF_KT * kst;           // [Dv][72]
-    const int vst = MF_KT + MF_VPAD;
+    bf16s* Vt = Ks + (size_t)MF_KT * kst;           // [Dv][68]
+    const int vst = MF_KT + 4;
     const int R = H / G;
     const int TT = 4 / HB, TQ = 16 * TT * NT;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -713,24 +705,23 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int dch = D / 8, vch = Dv / 8;
     // pages are a power of two: shifts, not divisions
     const int bsh = 31 - __clz(block_size), bmask = block_size - 1;
-    // Staging map: for K a thread owns ONE key per tile (key tid/4, every 4th
-    // 16-byte piece of its row); for V, cached page-wise transposed, it owns
-    // ONE run of 8 keys (run tid%8) of every 32nd value channel — both cost
-    // one page lookup per tile, and V^T reaches LDS in 16-byte pieces. The
-    // next tile's pieces are loaded into registers while this one is computed.
+    // Staging map: a thread owns ONE key per tile for K (key tid/4, every 4th
+    // 16-byte piece of its row) and one for V (key tid%64, every 4th piece),
+    // so a tile costs it two page lookups. The next tile's pieces are loaded
+    // into registers while the current tile is computed.
     constexpr int KC = MAXD / 2, VC = MAXDV / 2;
     const int kj = threadIdx.x >> 2, kc0 = threadIdx.x & 3;
-    const int vk = (threadIdx.x & 7) * 8, vd0 = threadIdx.x >> 3;   // keys vk..vk+7, channels vd0+32u
+    const int vj = threadIdx.x & 63, vc0 = threadIdx.x >> 6;
     uint4 kreg[KC], vreg[VC];
     auto fetch = [&](int kt) {
         const int k0 = kt * MF_KT;
         const int nk = min(MF_KT, block_last + 1 - k0);
-        const int keyk = k0 + kj, keyv = k0 + vk;
-        const bool okk = kj < nk, okv = vk < nk;
+        const int keyk = k0 + kj, keyv = k0 + vj;
+        const bool okk = kj < nk, okv = vj < nk;
         const int64_t sk_ = okk ? ((int64_t)bt[keyk >> bsh] << bsh) + (keyk & bmask) : 0;
+        const int64_t sv_ = okv ? ((int64_t)bt[keyv >> bsh] << bsh) + (keyv & bmask) : 0;
         const bf16s* kp = k_cache + (sk_ * G + g) * D;
-        const bf16s* vp = v_cache + (((int64_t)(okv ? bt[keyv >> bsh] : 0) * G + g) * Dv << bsh) +
-                          (keyv & bmask);
+        const bf16s* vp = v_cache + (sv_ * G + g) * Dv;
 #pragma unroll
         for (int u = 0; u < KC; ++u) {
             const int c = kc0 + 4 * u;
@@ -739,19 +730,9 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         }
 #pragma unroll
         for (int u = 0; u < VC; ++u) {
-            const int d = vd0 + 32 * u;
-            uint4 x = (okv && d < Dv) ? *reinterpret_cast<const uint4*>(vp + ((int64_t)d << bsh))
-                                      : make_uint4(0, 0, 0, 0);
-            if (okv && vk + 7 >= nk) {      // the sequence ends inside this run: stale keys -> 0
-                uint32_t w[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (vk + 2 * e >= nk) w[e] = 0;
-                    else if (vk + 2 * e + 1 >= nk) w[e] &= 0xffffu;
-                }
-                x = make_uint4(w[0], w[1], w[2], w[3]);
-            }
-            vreg[u] = x;
+            const int c = vc0 + 4 * u;
+            vreg[u] = (okv && c < vch) ? *reinterpret_cast<const uint4*>(vp + 8 * c)
+                                       : make_uint4(0, 0, 0, 0);
         }
     };
     if (split < nkt) fetch(split);
@@ -765,8 +746,15 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         }
 #pragma unroll
         for (int u = 0; u < VC; ++u) {
-            const int d = vd0 + 32 * u;
-            if (d < Dv) *reinterpret_cast<uint4*>(Vt + d * vst + vk) = vreg[u];
+            const int c = vc0 + 4 * u;
+            if (c < vch) {
+                const uint32_t w[4] = {vreg[u].x, vreg[u].y, vreg[u].z, vreg[u].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    Vt[(8 * c + 2 * e) * vst + vj] = (bf16s)(w[e] & 0xffffu);
+                    Vt[(8 * c + 2 * e + 1) * vst + vj] = (bf16s)(w[e] >> 16);
+                }
+            }
         }
         __syncthreads();
         if (kt + nsplit < nkt) fetch(kt + nsplit);
@@ -1347,7 +1335,7 @@ extern "C" int oa_group_rmsnorm(void* stream, const void* y, int64_t ys, int y_d
 extern "C" int oa_attn_prepare(void* stream, const void* qkv, int64_t qs, const void* bias, const void* qw,
                                const void* kw, void* q_out, void* k_cache, void* v_cache,
                                const void* slot_mapping, const void* cu, int B, int T, int H,
-                               int G, int D, int Dv, float eps, int dt, int block_size) {
+                               int G, int D, int Dv, float eps, int dt) {
     if (T <= 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (D % 8 == 0 && Dv % 8 == 0 && qs % 8 == 0 && (uintptr_t)qkv % 32 == 0 &&
@@ -1356,23 +1344,23 @@ extern "C" int oa_attn_prepare(void* stream, const void* qkv, int64_t qs, const 
             hipLaunchKernelGGL((attn_prepare_vec_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)qkv,
                                qs, (const float*)bias, (const float*)qw, (const float*)kw, (float*)q_out,
                                (float*)k_cache, (float*)v_cache, (const int*)slot_mapping, (const int*)cu,
-                               B, H, G, D, Dv, eps, block_size);
+                               B, H, G, D, Dv, eps);
         else
             hipLaunchKernelGGL((attn_prepare_vec_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const bf16s*)qkv,
                                qs, (const bf16s*)bias, (const bf16s*)qw, (const bf16s*)kw, (bf16s*)q_out,
                                (bf16s*)k_cache, (bf16s*)v_cache, (const int*)slot_mapping, (const int*)cu,
-                               B, H, G, D, Dv, eps, block_size);
+                               B, H, G, D, Dv, eps);
         HIP_CHECK_LAUNCH();
         return 0;
     }
     if (dt == 1)
         hipLaunchKernelGGL((attn_prepare_kernel<float>), dim3(T), dim3(256), 0, s, (const float*)qkv, qs,
                            (const float*)bias, (const float*)qw, (const float*)kw, (float*)q_out, (float*)k_cache,
-                           (float*)v_cache, (const int*)slot_mapping, (const int*)cu, B, H, G, D, Dv, eps, block_size);
+                           (float*)v_cache, (const int*)slot_mapping, (const int*)cu, B, H, G, D, Dv, eps);
     else
         hipLaunchKernelGGL((attn_prepare_kernel<bf16s>), dim3(T), dim3(256), 0, s, (const bf16s*)qkv, qs,
                            (const bf16s*)bias, (const bf16s*)qw, (const bf16s*)kw, (bf16s*)q_out, (bf16s*)k_cache,
-                           (bf16s*)v_cache, (const int*)slot_mapping, (const int*)cu, B, H, G, D, Dv, eps, block_size);
+                           (bf16s*)v_cache, (const int*)slot_mapping, (const int*)cu, B, H, G, D, Dv, eps);
     HIP_CHECK_LAUNCH();
     return 0;
 }
@@ -1403,7 +1391,7 @@ extern "C" int oa_attn_bias_geometry(int H, int G, int D, int Dv, int dt, int ma
         *TQ = 16 * (4 / attn_hb(R)) * attn_nt(D, Dv, max_chunk);
         *KT = MF_KT;
         *kstride = D + MF_KPAD;
-        *lds_bytes = (MF_KT * (D + MF_KPAD) + Dv * (MF_KT + MF_VPAD)) * 2;
+        *lds_bytes = (MF_KT * (D + MF_KPAD) + Dv * (MF_KT + 4)) * 2;
         return 0;
     }
     const int rb = std::min(R, 4 * ATT_MAXR);        // query heads per block
@@ -1452,7 +1440,6 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
     if (rc) return rc;
     if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return -104;
     hipStream_t s = (hipStream_t)stream;
-    if (block_size < 8 || (block_size & (block_size - 1)) != 0) return -108;
     if (attn_path(H, G, D, Dv, dt)) {
         const int R = H / G, HB = attn_hb(R);
         dim3 grid(ntiles, G * (R / HB), nsplit);

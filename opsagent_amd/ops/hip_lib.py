@@ -120,7 +120,7 @@ def _declare_mixers(lib: ctypes.CDLL) -> None:
     sigs = {
         "oa_causal_conv_seq": [p, p, i64, i, p, p, p, i64, p, p, p, p, i, i, i, i, i, i, i, i],
         "oa_group_rmsnorm": [p, p, i64, i, p, p, p, i, i, i, f, i],
-        "oa_attn_prepare": [p, p, i64, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, i],
+        "oa_attn_prepare": [p, p, i64, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i],
         "oa_attn_bias_geometry": [i, i, i, i, i, i, ip, ip, ip, ip],
         "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p,
                                i, i, i, i, i, i, i, f, i, i, i],

@@ -161,23 +161,22 @@ def attn_qkv_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm_w: 
                      v_cache: torch.Tensor, sb: SeqBatch) -> torch.Tensor:
     """qkv [T, >= H*D + G*D + G*Dv] (q | k | v columns first; bias over these
     columns is added first, if given). Norms q and k over their whole
-    projections, v per head; writes k, v to the paged cache (k as [blocks,
-    block_size, G, D], v page-wise transposed as [blocks, G, Dv, block_size]);
-    returns q [T, H, D]."""
+    projections, v per head; writes k, v to the paged cache; returns q
+    [T, H, D]."""
     T = qkv.shape[0]
     if not qkv.is_cuda:
         return torch_ref.attn_qkv_prepare(qkv, bias, q_norm_w, k_norm_w, H, G, D, Dv, eps,
                                           k_cache, v_cache, sb.slot_mapping)
     lib, hip = _lib()
     assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype
-    assert k_cache.shape[2:] == (G, D) and v_cache.shape[1:3] == (G, Dv)
+    assert k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, Dv)
     q = torch.empty(T, H, D, dtype=qkv.dtype, device=qkv.device)
     rc = lib.oa_attn_prepare(
         hip.current_stream_ptr(), qkv.data_ptr(), _rows(qkv),
         bias.data_ptr() if bias is not None else None, q_norm_w.data_ptr(),
         k_norm_w.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
         sb.slot_mapping.data_ptr(), sb.cu_t.data_ptr(), sb.num_seqs, T, H, G, D, Dv, eps,
-        _dt(qkv), k_cache.shape[1])
+        _dt(qkv))
     hip.check(rc, "oa_attn_prepare")
     return q
 
@@ -206,7 +205,7 @@ def attention_biased_paged(q: torch.Tensor, gate_logits: torch.Tensor, k_cache: 
     q.k*scale - slope_h*(i-j); head outputs times sigmoid(gate_logits[t, h]).
     q [T,H,D]; gate_logits [T,H] (may be a column slice). Returns [T, H*Dv]."""
     T, H, D = q.shape
-    nb, G, Dv, bs = v_cache.shape          # values are cached page-wise transposed
+    nb, bs, G, Dv = v_cache.shape
     if not q.is_cuda:
         return torch_ref.attention_biased_paged(q, gate_logits, k_cache, v_cache, sb.cu,
                                                 sb.past, sb.block_table, scale, slopes)

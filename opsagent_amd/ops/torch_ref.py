@@ -250,8 +250,7 @@ def attn_qkv_prepare(qkv, bias, q_norm_w, k_norm_w, H, G, D, Dv, eps, k_cache, v
     nb, bs = k_cache.shape[0], k_cache.shape[1]
     sm = slot_mapping.long()
     k_cache.view(nb * bs, G, D)[sm] = k.reshape(T, G, D).to(k_cache.dtype)
-    # values are cached page-wise transposed: [blocks, G, Dv, block_size]
-    v_cache[sm // bs, :, :, sm % bs] = v.to(v_cache.dtype)
+    v_cache.view(nb * bs, G, Dv)[sm] = v.to(v_cache.dtype)
     return q.reshape(T, H, D).to(qkv.dtype)
 
 
@@ -261,7 +260,7 @@ def attention_biased_paged(q, gate_logits, k_cache, v_cache, cu, past, block_tab
     keys 0..position, score = q.k*scale - slope_h*(i-j), each head's output
     times sigmoid(gate logit). q [T,H,D]; returns [T, H*Dv]."""
     T, H, D = q.shape
-    nb, G, Dv, bs = v_cache.shape          # page-wise transposed values
+    nb, bs, G, Dv = v_cache.shape
     out = torch.empty(T, H, Dv, dtype=q.dtype, device=q.device)
     rep = H // G
     for b in range(len(cu) - 1):
@@ -272,7 +271,7 @@ def attention_biased_paged(q, gate_logits, k_cache, v_cache, cu, past, block_tab
         nblk = (total + bs - 1) // bs
         blocks = block_table[b, :nblk].long()
         kk = k_cache[blocks].reshape(nblk * bs, G, D)[:total].float()
-        vv = v_cache[blocks].permute(0, 3, 1, 2).reshape(nblk * bs, G, Dv)[:total].float()
+        vv = v_cache[blocks].reshape(nblk * bs, G, Dv)[:total].float()
         kk = kk.repeat_interleave(rep, dim=1)
         vv = vv.repeat_interleave(rep, dim=1)
         qs = q[lo:hi].float()
