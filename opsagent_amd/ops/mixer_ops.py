@@ -268,6 +268,13 @@ def channel_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
             if Dv % (4 * c) == 0 and Dv // c >= 16 and pairs * c <= 512:
                 csplit = c
                 break
+    if D > 128 and Dv // csplit > 64:
+        # 256-row columns: more than 64 columns per block would hold two or
+        # four columns per lane pass and spill registers; split instead
+        for c in (2, 4):
+            if c >= csplit and Dv % (4 * c) == 0 and Dv // c <= 64:
+                csplit = c
+                break
     if csplit > 1:
         o_raw = torch.empty(T, H * Dv, dtype=torch.float32, device=q.device)
     rc = lib.oa_delta_rule_fused(
