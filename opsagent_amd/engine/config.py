@@ -178,7 +178,8 @@ def get_model_spec(name):
     if not isinstance(name, str):
         return name
     if name in HYBRID_REGISTRY:
-        return povazen_spec_from_dict(HYBRID_REGISTRY[name](), name=name)
+        cfg = HYBRID_REGISTRY[name]()
+        return ARCHITECTURE_PARSERS[cfg["architecture"]](cfg, name=name)
     if os.path.isdir(name) and os.path.exists(os.path.join(name, "config.json")):
         return load_spec_from_dir(name)
     if name not in MODEL_REGISTRY:
@@ -195,7 +196,10 @@ def get_model_spec(name):
 
 @dataclasses.dataclass
 class MixerSpec:
-    """One layer's token mixer. kind: "attention" | "channel_delta"."""
+    """One layer's token mixer. kind: "attention" (distance-penalty softmax
+    attention) | "channel_delta" (gated delta rule) | "rotary_window"
+    (rotary softmax attention with per-head query/key norm, an optional
+    sliding window and an optional sink term)."""
 
     kind: str
     heads: int
@@ -208,10 +212,19 @@ class MixerSpec:
     # checkpoint's tensor shapes give them (None => the mixer's default)
     decay_rank: Optional[int] = None
     gate_rank: Optional[int] = None
+    # rotary attention: rotated channels per head (0 = none), frequency base,
+    # wavelength-dependent rescaling {factor, low, high, original} or None
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional[dict] = None
+    # keys a query sees, itself included (None = all earlier keys)
+    window: Optional[int] = None
+    # a learned per-head term in the softmax denominator
+    sink: bool = False
 
     @property
     def has_kv(self) -> bool:
-        return self.kind == "attention"
+        return self.kind in ("attention", "rotary_window")
 
     @property
     def has_state(self) -> bool:
@@ -219,10 +232,32 @@ class MixerSpec:
 
 
 @dataclasses.dataclass
+class RouterSpec:
+    """Expert choice of a mixture-of-experts feed-forward. score: how router
+    logits become scores s ("sigmoid" | "softmax"); with `correction` the
+    ranking uses c = s + a learned vector while the mixing weights keep s;
+    `groups` > 1 cuts the experts into runs of neighbours rated
+    max1(c) + max2(c), of which the `keep` top-rated may be picked from;
+    w_j = scale * s_j / sum_k s_k over the `top` picked experts."""
+
+    experts: int
+    top: int
+    ff: int                          # an expert's inner size
+    score: str = "sigmoid"
+    correction: bool = True
+    groups: int = 1
+    keep: int = 1
+    scale: float = 1.0
+    shared_ff: int = 0               # inner size of the always-on expert (0 = none)
+
+
+@dataclasses.dataclass
 class HybridLayerSpec:
     mixer: MixerSpec
-    mlp_kind: Optional[str] = None   # None => the layer has no feed-forward
+    mlp_kind: Optional[str] = None   # None => no feed-forward; "dense" | "moe"
     mlp_ff: int = 0
+    mlp_act: str = "silu"            # dense feed-forward gate activation
+    router: Optional[RouterSpec] = None
 
 
 @dataclasses.dataclass
@@ -235,9 +270,13 @@ class HybridSpec:
     hidden_size: int
     layers: List[HybridLayerSpec]
     norm_eps: float
-    norm_groups: int
-    canon_taps: int
-    logit_softcap: float
+    norm_groups: int = 1
+    canon_taps: int = 0
+    logit_softcap: Optional[float] = None
+    # "post_canon": grouped RMS norm on sublayer outputs, sublayers read
+    # x + canon(x). "sandwich": a dynamic-tanh norm before and after every
+    # sublayer.
+    layer_style: str = "post_canon"
     max_seq_len: int = 1 << 20
     weights_path: Optional[str] = None
 
@@ -318,8 +357,106 @@ def povazen_config_dict(
             "vocab": vocab, "width": width}
 
 
+def vazilorn_spec_from_dict(cfg: dict, name: str = "vazilorn") -> HybridSpec:
+    """Parse a Vazilorn config.json dict: rotary sliding-window attention with
+    sinks between dynamic-tanh norms, dense or routed feed-forwards."""
+    layers = []
+    for entry in cfg["layers"]:
+        if entry["type"] != "attention":
+            raise ValueError(f"unknown Vazilorn layer type {entry['type']!r}")
+        m = entry["mixer"]
+        rot = m.get("rot") or {}
+        mask = m.get("mask") or {}
+        mixer = MixerSpec(
+            kind="rotary_window",
+            heads=int(m["heads"]),
+            kv_heads=int(m["kv_heads"]),
+            dim=int(m["dim"]),
+            vdim=int(m["vdim"]),
+            scale=float(m["scale"]) if "scale" in m else None,
+            rot_dims=int(rot.get("dims", 0)),
+            rot_base=float(rot.get("base", 10000.0)),
+            rot_scaling=dict(rot["scaling"]) if rot.get("scaling") else None,
+            window=int(mask["size"]) if mask.get("size") else None,
+            sink=True,
+        )
+        if mixer.heads % mixer.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if mixer.rot_dims % 2 or mixer.rot_dims > mixer.dim:
+            raise ValueError("rot.dims must be even and at most dim")
+        mlp = entry.get("mlp")
+        ls = HybridLayerSpec(mixer=mixer)
+        if mlp is not None:
+            kind = mlp.get("kind")
+            if kind == "dense":
+                ls.mlp_kind, ls.mlp_ff, ls.mlp_act = "dense", int(mlp["ff"]), "gelu_tanh"
+            elif kind == "moe":
+                r = mlp["router"]
+                grp = r.get("groups") or {}
+                shared = mlp.get("shared") or {}
+                ls.mlp_kind = "moe"
+                ls.router = RouterSpec(
+                    experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]),
+                    score="sigmoid", correction=True,
+                    groups=int(grp.get("count", 1)), keep=int(grp.get("keep", grp.get("count", 1))),
+                    scale=float(r.get("scale", 1.0)), shared_ff=int(shared.get("ff", 0)),
+                )
+                if ls.router.experts % ls.router.groups:
+                    raise ValueError("experts must be a multiple of groups.count")
+            else:
+                raise ValueError(f"unknown Vazilorn feed-forward kind {kind!r}")
+        layers.append(ls)
+    return HybridSpec(
+        name=name,
+        architecture="Vazilorn",
+        vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]),
+        layers=layers,
+        norm_eps=float(cfg["norm"]["eps"]),
+        layer_style="sandwich",
+    )
+
+
+def vazilorn_config_dict(
+    vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int,
+    vdim: int, ff: int, window: Optional[int] = 64, rot_dims: Optional[int] = None,
+    rot_base: float = 10000.0, rot_scaling: Optional[dict] = None, experts: int = 8,
+    top: int = 2, expert_ff: int = 64, groups: int = 2, keep: int = 1,
+    router_scale: float = 1.0, shared_ff: int = 0, eps: float = 1e-6,
+    scale: Optional[float] = None,
+) -> dict:
+    """A Vazilorn config.json dict from a layer pattern: 'd' = attention +
+    dense feed-forward, 'm' = attention + routed experts, 'a' = attention
+    alone."""
+    layers = []
+    for ch in pattern:
+        mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                 "scale": scale if scale is not None else dim ** -0.5,
+                 "rot": {"base": rot_base, "dims": dim if rot_dims is None else rot_dims}}
+        if rot_scaling:
+            mixer["rot"]["scaling"] = dict(rot_scaling)
+        if window:
+            mixer["mask"] = {"size": window}
+        if ch == "d":
+            mlp = {"kind": "dense", "ff": ff}
+        elif ch == "m":
+            mlp = {"kind": "moe", "expert": {"ff": expert_ff},
+                   "router": {"experts": experts, "top": top, "scale": router_scale,
+                              "groups": {"count": groups, "keep": keep}}}
+            if shared_ff:
+                mlp["shared"] = {"ff": shared_ff}
+        elif ch == "a":
+            mlp = None
+        else:
+            raise ValueError(f"unknown layer letter {ch!r}")
+        layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Vazilorn", "layers": layers, "norm": {"eps": eps},
+            "vocab": vocab, "width": width}
+
+
 # config.json "architecture" -> parser
-ARCHITECTURE_PARSERS = {"Povazen": povazen_spec_from_dict}
+ARCHITECTURE_PARSERS = {"Povazen": povazen_spec_from_dict,
+                        "Vazilorn": vazilorn_spec_from_dict}
 
 # named hybrid configurations (random-weight benchmarking and tests)
 HYBRID_REGISTRY = {
@@ -336,6 +473,25 @@ HYBRID_REGISTRY = {
     "povazen-4l4k": lambda: povazen_config_dict(
         vocab=2048, width=4096, pattern="dada", heads=32, kv_heads=8, dim=128,
         vdim=128, ff=14336, delta_heads=32),
+    # CPU-test size
+    "vazilorn-tiny": lambda: vazilorn_config_dict(
+        vocab=512, width=64, pattern="dma", heads=4, kv_heads=2, dim=16, vdim=8,
+        ff=128, window=24, rot_dims=8, experts=8, top=2, expert_ff=32, groups=2,
+        keep=1, router_scale=1.5, shared_ff=48),
+    # GPU-smoke size
+    "vazilorn-micro": lambda: vazilorn_config_dict(
+        vocab=2048, width=1024, pattern="dmdm", heads=8, kv_heads=2, dim=128,
+        vdim=128, ff=2816, window=512, experts=16, top=4, expert_ff=512, groups=4,
+        keep=2, router_scale=2.0, shared_ff=512,
+        rot_scaling={"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}),
+    # dense layer shapes of an ~8B-class model at 4 layers (speed beside
+    # llama3 layers of equal width)
+    "vazilorn-4l4k": lambda: vazilorn_config_dict(
+        vocab=2048, width=4096, pattern="dddd", heads=32, kv_heads=8, dim=128,
+        vdim=128, ff=14336, window=1024),
+    "vazilorn-4l2k": lambda: vazilorn_config_dict(
+        vocab=2048, width=2048, pattern="dddd", heads=16, kv_heads=4, dim=128,
+        vdim=128, ff=8192, window=1024),
 }
 
 
@@ -362,8 +518,13 @@ def load_spec_from_dir(path: str):
 
 def apply_tensor_shapes(spec: HybridSpec, shapes: dict) -> HybridSpec:
     """Fill the sizes that only tensor shapes give (name -> shape): the inner
-    ranks of the low-rank decay and output-gate projections."""
+    ranks of the low-rank decay and output-gate projections, whether an
+    attention mixer carries a sink and a router a correction."""
     for i, layer in enumerate(spec.layers):
+        if layer.mixer.kind == "rotary_window":
+            layer.mixer.sink = f"l{i}.mix.sink" in shapes
+        if layer.router is not None:
+            layer.router.correction = f"l{i}.mlp.correction" in shapes
         a1, g1 = shapes.get(f"l{i}.mix.a1"), shapes.get(f"l{i}.mix.g1")
         if a1 is not None:
             layer.mixer.decay_rank = int(a1[0])

@@ -1,11 +1,18 @@
-"""Hybrid decoder (the Povazen design): a per-layer choice of token mixer —
-softmax attention with a linear distance penalty, or a gated delta rule with
-per-channel decay — around a float32 residual stream.
+"""Hybrid decoders: a per-layer choice of token mixer and feed-forward
+around a float32 residual stream, in two layer styles.
 
+"post_canon" (the Povazen design): softmax attention with a linear distance
+penalty, or a gated delta rule with per-channel decay.
 Layer:  x <- x + norm1(mixer(h)),  h = x + canon(x);  x <- x + norm2(ff(x)).
 The norms sit on the sublayer OUTPUTS (grouped RMS norm); the sublayers read
 the raw stream. canon is a causal per-channel convolution over time whose
 last inputs are carried per sequence, like the recurrent state.
+
+"sandwich" (the Vazilorn design): rotary sliding-window attention with a
+sink term, dense gelu or routed-expert feed-forwards.
+Layer:  x <- x + post1(mixer(pre1(x)));  x <- x + post2(ff(pre2(x))),
+every norm elementwise: tanh(a x) w + b with one scalar a, no statistics
+over channels.
 
 The mixers are modules of their own (BiasedAttentionMixer,
 ChannelDeltaMixer) with every constant a constructor argument, built on the
@@ -92,6 +99,62 @@ class BiasedAttentionMixer(nn.Module):
         return ops.linear(ctx, self.o_w)
 
 
+class RotaryWindowAttentionMixer(nn.Module):
+    """Causal softmax attention with rotary positions. Order of operations
+    on a query or key head: RMS norm over the head's `dim` channels (weight
+    [dim], one per projection, the same for every head), then rotation of
+    channels (2i, 2i+1), i < rot_dims/2, by position * f_i with
+    f_i = rot_base^(-2i/rot_dims), optionally rescaled by wavelength.
+    Visible keys: the last `window` positions up to the query (None: the
+    whole past). With sink=True head h's normaliser is
+    sum_j exp(score_j) + exp(sink_h), sink_h learned. Norm weights, sinks,
+    angles, scores and softmax weights are float32.
+
+    Fused projection rows: q | k | v."""
+
+    def __init__(self, hidden: int, m: MixerSpec, eps: float, dtype, gen):
+        super().__init__()
+        self.H, self.G, self.D, self.Dv = m.heads, m.kv_heads, m.dim, m.vdim
+        self.eps = eps
+        self.scale = float(m.scale) if m.scale is not None else m.dim ** -0.5
+        self.window = int(m.window) if m.window else None
+        dev = gen.device
+        n = self.H * self.D + self.G * (self.D + self.Dv)
+        self.proj_w = _param(_rand(gen, n, hidden, std=1.0 / math.sqrt(hidden), dtype=dtype))
+        self.q_norm_w = _param(1.0 + 0.1 * _rand(gen, self.D))
+        self.k_norm_w = _param(1.0 + 0.1 * _rand(gen, self.D))
+        self.sinks = _param(_rand(gen, self.H)) if m.sink else None
+        self.o_w = _param(_rand(gen, hidden, self.H * self.Dv,
+                                std=1.0 / math.sqrt(self.H * self.Dv), dtype=dtype))
+        self.register_buffer(
+            "inv_freq", mx.rotary_inv_freq(m.rot_dims, m.rot_base, m.rot_scaling).to(dev),
+            persistent=False)
+
+    def kv_shape(self):
+        return (self.G, self.D, self.Dv)
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return {}
+
+    def forward(self, h, sb: mx.SeqBatch, kv, state) -> torch.Tensor:
+        k_cache, v_cache = kv
+        proj = ops.linear(h, self.proj_w)                     # [T, q|k|v]
+        q = mx.attn_rope_prepare(proj, self.q_norm_w, self.k_norm_w, self.inv_freq,
+                                 self.H, self.G, self.D, self.Dv, self.eps,
+                                 k_cache, v_cache, sb)
+        ctx = mx.attention_paged(q, k_cache, v_cache, sb, self.scale,
+                                 window=self.window, sinks=self.sinks)
+        return ops.linear(ctx, self.o_w)
+
+    def load(self, get, put, p: str) -> None:
+        put(self.proj_w, [get(p + "q"), get(p + "k"), get(p + "v")])
+        put(self.q_norm_w, [get(p + "q.norm")])
+        put(self.k_norm_w, [get(p + "k.norm")])
+        if self.sinks is not None:
+            put(self.sinks, [get(p + "sink")])
+        put(self.o_w, [get(p + "o")])
+
+
 class ChannelDeltaMixer(nn.Module):
     """Gated delta rule with one decay per head and key channel.
 
@@ -152,15 +215,17 @@ class ChannelDeltaMixer(nn.Module):
         return ops.linear(y, self.o_w)
 
 
-MIXERS = {"attention": BiasedAttentionMixer, "channel_delta": ChannelDeltaMixer}
+MIXERS = {"attention": BiasedAttentionMixer, "channel_delta": ChannelDeltaMixer,
+          "rotary_window": RotaryWindowAttentionMixer}
 
 
 class GatedMLP(nn.Module):
-    """down(silu(gate x) * (up x)); gate|up fused."""
+    """down(act(gate x) * (up x)); gate|up fused; act "silu" | "gelu_tanh"."""
 
-    def __init__(self, hidden: int, ff: int, dtype, gen):
+    def __init__(self, hidden: int, ff: int, dtype, gen, act: str = "silu"):
         super().__init__()
         self.ff = ff
+        self.act = act
         self.gate_up_w = _param(_rand(gen, 2 * ff, hidden, std=1.0 / math.sqrt(hidden), dtype=dtype))
         self.down_w = _param(_rand(gen, hidden, ff, std=1.0 / math.sqrt(ff), dtype=dtype))
 
@@ -170,10 +235,14 @@ class GatedMLP(nn.Module):
             x.is_cuda and x.dtype == torch.bfloat16 and K % 8 == 0 and self.ff % 8 == 0
             and (ops._gemv_m_ok(M) or ops._bf16_mfma_ok(M, K, gateup=True))
         ):
-            act = ops.gateup_silu(x, self.gate_up_w, self.ff)   # fused decode GEMV
+            act = ops.gateup_act(x, self.gate_up_w, self.ff, self.act)   # fused decode GEMV
         else:
-            act = mx.silu_mul_rows(ops.linear(x, self.gate_up_w), self.ff)
+            act = mx.act_mul_rows(ops.linear(x, self.gate_up_w), self.ff, self.act)
         return ops.linear(act, self.down_w)
+
+    def load(self, get, put, p: str) -> None:
+        put(self.gate_up_w, [get(p + "gate"), get(p + "up")])
+        put(self.down_w, [get(p + "down")])
 
 
 class HybridLayer(nn.Module):
@@ -209,8 +278,81 @@ class HybridLayer(nn.Module):
         return x
 
 
+class DyTNorm(nn.Module):
+    """Dynamic-tanh norm tanh(a x) w + b: weight and bias per channel, one
+    scalar a; float32 parameters whatever the model's type."""
+
+    def __init__(self, width: int, gen, alpha: float = 0.5):
+        super().__init__()
+        dev = gen.device
+        self.w = _param(torch.ones(width, device=dev) + 0.05 * _rand(gen, width))
+        self.b = _param(0.02 * _rand(gen, width))
+        self.alpha = _param(torch.full((1,), float(alpha), device=dev))
+
+    def params(self):
+        return (self.w, self.b, self.alpha)
+
+    def load(self, get, put, name: str) -> None:
+        put(self.w, [get(name)])
+        put(self.b, [get(name + ".b")])
+        put(self.alpha, [get(name + ".alpha").reshape(1)])
+
+
+class SandwichLayer(nn.Module):
+    """x <- x + post1(mixer(pre1(x)));  x <- x + post2(ff(pre2(x))) with
+    dynamic-tanh norms. The add after a sublayer and the norm before the
+    next one (also the next layer's) are one launch: forward takes the
+    already-normed mixer input and returns the next layer's."""
+
+    def __init__(self, spec: HybridSpec, ls: HybridLayerSpec, dtype, gen):
+        super().__init__()
+        C = spec.hidden_size
+        self.dtype = dtype
+        self.pre1, self.post1 = DyTNorm(C, gen), DyTNorm(C, gen)
+        self.mixer = MIXERS[ls.mixer.kind](C, ls.mixer, spec.norm_eps, dtype, gen)
+        self.mlp = None
+        if ls.mlp_kind == "dense":
+            self.mlp = GatedMLP(C, ls.mlp_ff, dtype, gen, act=ls.mlp_act)
+        elif ls.mlp_kind == "moe":
+            from opsagent_amd.engine.moe import RoutedExperts
+
+            self.mlp = RoutedExperts(C, ls.router, dtype, gen)
+        self.routed = ls.mlp_kind == "moe"
+        if self.mlp is not None:
+            self.pre2, self.post2 = DyTNorm(C, gen), DyTNorm(C, gen)
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return dict(self.mixer.state_shapes())
+
+    def first_norm(self):
+        return self.pre1.params()
+
+    def forward(self, x, h, sb: mx.SeqBatch, kv, state, next_norm):
+        """x: float32 residual [T, C] (updated in place); h = pre1(x).
+        next_norm: the following layer's first norm (None after the last
+        layer). Returns (x, next layer's h or None)."""
+        y = self.mixer(h, sb, kv, state)
+        if self.mlp is None:
+            return x, mx.dyt_norm(x, next_norm, self.dtype, y=y, post=self.post1.params())
+        h2 = mx.dyt_norm(x, self.pre2.params(), self.dtype, y=y, post=self.post1.params())
+        m = self.mlp(h2, decode=sb.max_chunk == 1) if self.routed else self.mlp(h2)
+        return x, mx.dyt_norm(x, next_norm, self.dtype, y=m, post=self.post2.params())
+
+    def load(self, get, put, p: str) -> None:
+        self.pre1.load(get, put, p + "norm1")
+        self.post1.load(get, put, p + "norm1b")
+        self.mixer.load(get, put, p + "mix.")
+        if self.mlp is not None:
+            self.pre2.load(get, put, p + "norm2")
+            self.post2.load(get, put, p + "norm2b")
+            self.mlp.load(get, put, p + "mlp.")
+
+
+LAYER_STYLES = {"post_canon": HybridLayer, "sandwich": SandwichLayer}
+
+
 class HybridForCausalLM(nn.Module):
-    """Embedding -> hybrid layers -> grouped RMS norm -> head -> soft cap."""
+    """Embedding -> hybrid layers -> final norm -> head (-> soft cap)."""
 
     def __init__(self, spec: HybridSpec, dtype: torch.dtype = torch.bfloat16,
                  device: str = "cpu", seed: int = 1234):
@@ -222,10 +364,14 @@ class HybridForCausalLM(nn.Module):
         gen = torch.Generator(device=device).manual_seed(seed)
         C = spec.hidden_size
         self.embed = _param(_rand(gen, spec.vocab_size, C, dtype=dtype))
+        self.sandwich = spec.layer_style == "sandwich"
         self.layers = nn.ModuleList(
-            [HybridLayer(spec, ls, dtype, gen) for ls in spec.layers]
+            [LAYER_STYLES[spec.layer_style](spec, ls, dtype, gen) for ls in spec.layers]
         )
-        self.final_norm_w = _param(torch.ones(C, dtype=dtype, device=device))
+        if self.sandwich:
+            self.final_norm = DyTNorm(C, gen)
+        else:
+            self.final_norm_w = _param(torch.ones(C, dtype=dtype, device=device))
         self.lm_head = _param(_rand(gen, spec.vocab_size, C, std=1.0 / math.sqrt(C), dtype=dtype))
         self.vocab_local = spec.vocab_size
         self.to(device)
@@ -243,6 +389,15 @@ class HybridForCausalLM(nn.Module):
         sb = fb.seq_batch
         assert sb is not None and state is not None, "hybrid models run flat multi-sequence steps"
         x = mx.embed_rows(self.embed, fb.input_ids)
+        if self.sandwich:
+            n = len(self.layers)
+            h = mx.dyt_norm(x, self.layers[0].first_norm(), self.dtype)
+            for i, layer in enumerate(self.layers):
+                nxt = self.layers[i + 1].first_norm() if i + 1 < n else None
+                x, h = layer(x, h, sb, kv_caches[i], state[i], nxt)
+                if self.trace_layers is not None:
+                    self.trace_layers.append(x.clone())
+            return x
         for i, layer in enumerate(self.layers):
             x = layer(x, sb, kv_caches[i], state[i])
             if self.trace_layers is not None:
@@ -250,10 +405,17 @@ class HybridForCausalLM(nn.Module):
         return x  # float32 residual [T, C]; compute_logits norms the rows it needs
 
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
-        """hidden: float32 residual rows. Returns float32 soft-capped logits."""
-        _, normed = mx.group_rms_norm(hidden, self.final_norm_w, self.spec.norm_groups,
-                                      self.spec.norm_eps, residual=None)
-        return mx.softcap(ops.linear(normed, self.lm_head), self.spec.logit_softcap)
+        """hidden: float32 residual rows. Returns float32 logits (soft-capped
+        if the design caps them)."""
+        if self.sandwich:
+            normed = mx.dyt_norm(hidden.contiguous(), self.final_norm.params(), self.dtype)
+        else:
+            _, normed = mx.group_rms_norm(hidden, self.final_norm_w, self.spec.norm_groups,
+                                          self.spec.norm_eps, residual=None)
+        logits = ops.linear(normed, self.lm_head)
+        if self.spec.logit_softcap is None:
+            return logits.float()
+        return mx.softcap(logits, self.spec.logit_softcap)
 
     # -- checkpoint names ----------------------------------------------------
     @torch.no_grad()
@@ -268,7 +430,8 @@ class HybridForCausalLM(nn.Module):
             t = torch.cat([p.reshape(p.shape[0], -1) if param.dim() == 2 else p.reshape(-1)
                            for p in parts], 0)
             assert tuple(t.shape) == tuple(param.shape), (tuple(t.shape), tuple(param.shape))
-            param.data.copy_(t.to(device=dev, dtype=dtype))
+            # float32 parameters (norms, sinks, routers) stay float32
+            param.data.copy_(t.to(device=dev, dtype=param.dtype))
             n += len(parts)
 
         def get(name):
@@ -277,8 +440,13 @@ class HybridForCausalLM(nn.Module):
             return tensors[name]
 
         put(self.embed, [get("embed")])
-        put(self.final_norm_w, [get("final.norm")])
         put(self.lm_head, [get("head")])
+        if self.sandwich:
+            self.final_norm.load(get, put, "final.norm")
+            for i, layer in enumerate(self.layers):
+                layer.load(get, put, f"l{i}.")
+            return n
+        put(self.final_norm_w, [get("final.norm")])
         for i, layer in enumerate(self.layers):
             p = f"l{i}."
             put(layer.norm1_w, [get(p + "norm1")])

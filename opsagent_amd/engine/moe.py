@@ -172,3 +172,119 @@ class MoEMLP(nn.Module):
             return self.forward(x)
         finally:
             self._force_loop = False
+
+
+class RoutedExperts(nn.Module):
+    """Mixture of gated feed-forwards with a score-and-choose router whose
+    every constant is a RouterSpec field: sigmoid (or softmax) scores, a
+    learned correction that enters the CHOICE only, group-limited choice,
+    weights normalised over the chosen experts and scaled, an optional
+    always-on shared expert. Router logits, scores and weights are float32.
+
+    Expert weights are stacked: w13 [E, 2I, C] (gate rows, then up rows) and
+    w2 [E, C, I]. Few (token, expert) pairs run through two static-shaped
+    launches without host sync (hipGraph-capturable); prompt-sized batches
+    are sorted by expert and run one library GEMM pair per used expert.
+    """
+
+    def __init__(self, hidden: int, r, dtype: torch.dtype, gen: torch.Generator,
+                 act: str = "silu"):
+        super().__init__()
+        if get_tp_size() != 1:
+            raise NotImplementedError("routed experts run at tensor-parallel size 1")
+        from opsagent_amd.engine.hybrid import GatedMLP, _param, _rand
+
+        self.r, self.act, self.hidden = r, act, hidden
+        E, I = r.experts, r.ff
+        self.router_w = _param(_rand(gen, E, hidden, std=hidden ** -0.5))
+        self.correction = _param(0.1 * _rand(gen, E)) if r.correction else None
+        self.w13 = _param(_rand(gen, E, 2 * I, hidden, std=hidden ** -0.5, dtype=dtype))
+        self.w2 = _param(_rand(gen, E, hidden, I, std=I ** -0.5, dtype=dtype))
+        self.shared = GatedMLP(hidden, r.shared_ff, dtype, gen, act=act) if r.shared_ff else None
+        # weight bytes one launch pair may stream through the pair kernels
+        self.pair_budget = 64 << 20
+        self.force_path = None     # "pairs" | "sorted" (tests)
+
+    def route(self, x: torch.Tensor):
+        from opsagent_amd.ops import mixer_ops as mx
+
+        logits = F.linear(x.float(), self.router_w)
+        return mx.route_topk(logits, self.correction, self.r.top, self.r.groups, self.r.keep,
+                             self.r.scale, self.r.score)
+
+    def forward(self, x: torch.Tensor, decode: bool = False) -> torch.Tensor:
+        """decode: the step holds one token per sequence; such batches stay on
+        the static-shaped pair kernels up to 2048 pairs, so the step can be
+        captured in a hipGraph."""
+        T, C = x.shape
+        idx, wts = self.route(x)
+        P, I = T * self.r.top, self.r.ff
+        esz = 4 if x.dtype == torch.float32 else 2
+        pairs = (P <= 64 or P * 3 * I * C * esz <= self.pair_budget
+                 or (decode and P <= 2048))
+        if self.force_path is not None:
+            pairs = self.force_path == "pairs"
+        if pairs:
+            out = self._pairs(x, idx, wts)
+        else:
+            out = self._sorted(x, idx, wts)
+        if self.shared is not None:
+            out = out + self.shared(x)
+        return out
+
+    def _pairs(self, x, idx, wts):
+        from opsagent_amd.ops import mixer_ops as mx
+
+        T, C = x.shape
+        I, top = self.r.ff, self.r.top
+        if (x.is_cuda and x.dtype == torch.bfloat16 and self.act == "silu"
+                and C % 16 == 0 and I % 16 == 0 and self.force_path is None):
+            # the framework's grouped expert GEMV kernels (pair- or expert-major)
+            flat_t = torch.arange(T, device=x.device, dtype=torch.int32).repeat_interleave(top)
+            y = ops.moe_grouped_mlp(x.contiguous(), self.w13, None, self.w2, None,
+                                    idx.reshape(-1), flat_t.contiguous(),
+                                    wts.reshape(-1).contiguous(), I, False,
+                                    num_experts=self.r.experts)
+            return y.view(T, top, C).float().sum(1).to(x.dtype)
+        return mx.moe_pairs_mlp(x.contiguous(), self.w13, self.w2, idx, wts, self.act)
+
+    def _sorted(self, x, idx, wts):
+        from opsagent_amd.ops import mixer_ops as mx
+
+        T, C = x.shape
+        top, I = self.r.top, self.r.ff
+        flat_e = idx.reshape(-1).long()
+        order = torch.argsort(flat_e, stable=True)
+        tok = torch.div(order, top, rounding_mode="floor")
+        w_sorted = wts.reshape(-1)[order]
+        # ONE host sync for the whole dispatch
+        counts = torch.bincount(flat_e, minlength=self.r.experts).cpu().tolist()
+        xs = x.index_select(0, tok)
+        ys = torch.empty(T * top, C, dtype=torch.float32, device=x.device)
+        start = 0
+        for e, c in enumerate(counts):
+            if c == 0:
+                continue
+            gu = ops.linear(xs[start : start + c], self.w13[e])
+            a = mx.act_mul_rows(gu, I, self.act)
+            ys[start : start + c] = ops.linear(a, self.w2[e]).float()
+            start += c
+        ys *= w_sorted.unsqueeze(1)
+        # back to (token, choice) order: a token's experts are summed in its
+        # own order whatever else the batch holds
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(order.numel(), device=order.device)
+        return ys.index_select(0, inv).view(T, top, C).sum(1).to(x.dtype)
+
+    def load(self, get, put, p: str) -> None:
+        E = self.r.experts
+        put(self.router_w, [get(p + "router")])
+        if self.correction is not None:
+            put(self.correction, [get(p + "correction")])
+        w13 = torch.stack([torch.cat([get(f"{p}e{k}.gate"), get(f"{p}e{k}.up")], 0)
+                           for k in range(E)])
+        w2 = torch.stack([get(f"{p}e{k}.down") for k in range(E)])
+        self.w13.data.copy_(w13.to(self.w13.device, self.w13.dtype))
+        self.w2.data.copy_(w2.to(self.w2.device, self.w2.dtype))
+        if self.shared is not None:
+            self.shared.load(get, put, p + "shared.")

@@ -474,6 +474,26 @@ def gateup_silu(x: torch.Tensor, gate_up_w: torch.Tensor, i_local: int) -> torch
     return silu_mul(gate.contiguous(), up.contiguous())
 
 
+def gateup_act(x: torch.Tensor, gate_up_w: torch.Tensor, i_local: int,
+               act: str = "silu") -> torch.Tensor:
+    """act(x @ gate^T) * (x @ up^T), act "silu" | "gelu_tanh", for decode-sized
+    bf16 batches: one fused GEMV launch."""
+    if act == "silu":
+        return gateup_silu(x, gate_up_w, i_local)
+    from opsagent_amd.ops import hip_lib
+
+    M = x.numel() // x.shape[-1]
+    assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and act == "gelu_tanh"
+    lib = hip_lib.get_lib()
+    out = torch.empty(*x.shape[:-1], i_local, dtype=x.dtype, device=x.device)
+    rc = lib.oa_gemv_gateup_act(
+        hip_lib.current_stream_ptr(), x.data_ptr(), gate_up_w.data_ptr(),
+        out.data_ptr(), M, i_local, x.shape[-1], 1,
+    )
+    hip_lib.check(rc, "oa_gemv_gateup_act")
+    return out
+
+
 def kv_cache_write(
     k_cache: torch.Tensor,
     v_cache: torch.Tensor,

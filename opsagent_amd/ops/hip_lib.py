@@ -45,6 +45,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.oa_rope_kv.restype = i
     lib.oa_gemv_gateup.argtypes = [p, p, p, p, i, i, i]
     lib.oa_gemv_gateup.restype = i
+    lib.oa_gemv_gateup_act.argtypes = [p, p, p, p, i, i, i, i]
+    lib.oa_gemv_gateup_act.restype = i
     lib.oa_gemv.argtypes = [p, p, p, p, i, i, i]
     lib.oa_gemv.restype = i
     lib.oa_gemv_ex.argtypes = [p, p, p, p, p, p, i, i, i, f, i]
@@ -122,8 +124,15 @@ def _declare_mixers(lib: ctypes.CDLL) -> None:
         "oa_group_rmsnorm": [p, p, i64, i, p, p, p, i, i, i, f, i],
         "oa_attn_prepare": [p, p, i64, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i],
         "oa_attn_bias_geometry": [i, i, i, i, i, i, ip, ip, ip, ip],
-        "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p,
-                               i, i, i, i, i, i, i, f, i, i, i],
+        "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p, p,
+                               i, i, i, i, i, i, i, f, i, i, i, i],
+        "oa_dyt_norm": [p, p, i64, i, p, p, p, p, p, p, p, p, i, i, i],
+        "oa_attn_rope_prepare": [p, p, i64, p, p, p, i, p, p, p, p, p, p, p, i, i,
+                                 i, i, i, i, f, i],
+        "oa_act_mul_rows": [p, p, p, i64, i, i, i],
+        "oa_route_topk": [p, p, p, p, p, i, i, i, i, i, f, i],
+        "oa_moe_pairs_gateup": [p, p, p, p, p, i, i, i, i, i, i, i],
+        "oa_moe_pairs_down": [p, p, p, p, p, p, i, i, i, i, i, i],
         "oa_delta_rule_fused": [p, p, i64, p, i64, p, i64, p, i64, p, i64, p, p, p, p, i64,
                                 p, p, p, p, p, p, i, i, i, i, i, i, f, i, i],
         "oa_softcap": [p, p, p, i64, f, i],

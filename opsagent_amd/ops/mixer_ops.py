@@ -198,23 +198,33 @@ def attn_geometry(H: int, G: int, D: int, Dv: int, dt: int, max_chunk: int) -> T
     return _GEOM[key]
 
 
-def attention_biased_paged(q: torch.Tensor, gate_logits: torch.Tensor, k_cache: torch.Tensor,
-                           v_cache: torch.Tensor, sb: SeqBatch, scale: float,
-                           slopes: torch.Tensor) -> torch.Tensor:
-    """Causal softmax attention over each sequence's cached keys with score
-    q.k*scale - slope_h*(i-j); head outputs times sigmoid(gate_logits[t, h]).
-    q [T,H,D]; gate_logits [T,H] (may be a column slice). Returns [T, H*Dv]."""
+def attention_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    sb: SeqBatch, scale: float, slopes: Optional[torch.Tensor] = None,
+                    gate_logits: Optional[torch.Tensor] = None,
+                    window: Optional[int] = None,
+                    sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal softmax attention over each sequence's cached keys, score
+    q.k*scale. Options, each a parameter: `slopes` [H] float32 subtracts
+    slope_h*(i-j); `window` hides keys with i - j >= window; `sinks` [H]
+    float32 enlarges head h's softmax normaliser by exp(sink_h) and leaves
+    the numerator alone;
+    `gate_logits` [T,H] (may be a column slice) scales each head's output by
+    its sigmoid. q [T,H,D]. Returns [T, H*Dv]."""
     T, H, D = q.shape
     nb, bs, G, Dv = v_cache.shape
+    window = int(window) if window else 0
     if not q.is_cuda:
-        return torch_ref.attention_biased_paged(q, gate_logits, k_cache, v_cache, sb.cu,
-                                                sb.past, sb.block_table, scale, slopes)
+        return torch_ref.attention_paged(q, k_cache, v_cache, sb.cu, sb.past, sb.block_table,
+                                         scale, slopes, gate_logits, window or None, sinks)
     lib, hip = _lib()
     dt = _dt(q)
     TQ, KT = attn_geometry(H, G, D, Dv, dt, sb.max_chunk)
     ntiles = sum((sb.cu[b + 1] - sb.cu[b] + TQ - 1) // TQ for b in range(sb.num_seqs))
     # few tiles and long contexts: split the keys over blocks to fill the chip
-    nkt = max(1, (sb.max_total + KT - 1) // KT)
+    reach = sb.max_total
+    if window:
+        reach = min(reach, window + min(sb.max_chunk, TQ) + KT)
+    nkt = max(1, (reach + KT - 1) // KT)
     nsplit = 1
     if ntiles * G < 256 and nkt >= 8:
         nsplit = int(min(nkt // 4, max(1, 512 // max(1, ntiles * G)), 64))
@@ -223,16 +233,191 @@ def attention_biased_paged(q: torch.Tensor, gate_logits: torch.Tensor, k_cache: 
     if nsplit > 1:
         part_o = torch.empty(T * H * nsplit, Dv, dtype=torch.float32, device=q.device)
         part_ml = torch.empty(T * H * nsplit, 2, dtype=torch.float32, device=q.device)
-    assert slopes.dtype == torch.float32 and q.is_contiguous()
+    assert q.is_contiguous()
+    assert slopes is None or (slopes.dtype == torch.float32 and slopes.numel() == H)
+    assert sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == H
+                             and sinks.is_contiguous())
     rc = lib.oa_attn_bias_paged(
-        hip.current_stream_ptr(), q.data_ptr(), gate_logits.data_ptr(), _rows(gate_logits),
+        hip.current_stream_ptr(), q.data_ptr(),
+        gate_logits.data_ptr() if gate_logits is not None else None,
+        _rows(gate_logits) if gate_logits is not None else 0,
         k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
         part_o.data_ptr() if part_o is not None else None,
         part_ml.data_ptr() if part_ml is not None else None,
         sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.block_table.data_ptr(),
-        sb.block_table.shape[1], bs, slopes.data_ptr(), T, sb.num_seqs, ntiles, H, G, D, Dv,
-        float(scale), nsplit, dt, sb.max_chunk)
+        sb.block_table.shape[1], bs, slopes.data_ptr() if slopes is not None else None,
+        sinks.data_ptr() if sinks is not None else None,
+        T, sb.num_seqs, ntiles, H, G, D, Dv,
+        float(scale), nsplit, dt, sb.max_chunk, window)
     hip.check(rc, "oa_attn_bias_paged")
+    return out
+
+
+def attention_biased_paged(q: torch.Tensor, gate_logits: torch.Tensor, k_cache: torch.Tensor,
+                           v_cache: torch.Tensor, sb: SeqBatch, scale: float,
+                           slopes: torch.Tensor) -> torch.Tensor:
+    """attention_paged with a distance penalty and an output gate."""
+    return attention_paged(q, k_cache, v_cache, sb, scale, slopes=slopes,
+                           gate_logits=gate_logits)
+
+
+def dyt_norm(residual: torch.Tensor, nxt: Optional[Tuple[torch.Tensor, ...]], out_dtype,
+             y: Optional[torch.Tensor] = None,
+             post: Optional[Tuple[torch.Tensor, ...]] = None) -> Optional[torch.Tensor]:
+    """Dynamic-tanh norm dyt(x; w, b, a) = tanh(a x) * w + b, computed in
+    float32; a norm is the tuple (w [C], b [C], a [1]) of float32 tensors.
+    With y [T, C] and post: residual (float32 [T, C]) += dyt(y; post) in
+    place. With nxt: returns dyt(residual; nxt) in out_dtype — one launch
+    for the add after a sublayer and the norm before the next one."""
+    T, C = residual.shape
+    assert residual.dtype == torch.float32 and residual.is_contiguous()
+    assert (y is None) == (post is None) and (y is not None or nxt is not None)
+    if not residual.is_cuda:
+        return torch_ref.dyt_norm(y, post, residual, nxt, out_dtype)
+    lib, hip = _lib()
+    for t in (post or ()) + (nxt or ()):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    out = torch.empty(T, C, dtype=out_dtype, device=residual.device) if nxt is not None else None
+    pw, pb, pa = (t.data_ptr() for t in post) if post is not None else (None, None, None)
+    nw, nb, na = (t.data_ptr() for t in nxt) if nxt is not None else (None, None, None)
+    rc = lib.oa_dyt_norm(
+        hip.current_stream_ptr(), y.data_ptr() if y is not None else None,
+        _rows(y) if y is not None else 0, _dt(y) if y is not None else 1, pw, pb, pa,
+        residual.data_ptr(), nw, nb, na, out.data_ptr() if out is not None else None,
+        _dt(out) if out is not None else 1, T, C)
+    hip.check(rc, "oa_dyt_norm")
+    return out
+
+
+def rotary_inv_freq(dims: int, base: float, scaling: Optional[dict] = None) -> torch.Tensor:
+    """float32 [dims/2] rotation frequencies base^(-2i/dims). `scaling`
+    {factor, low, high, original} slows long waves: a wavelength below
+    original/high keeps its frequency, one above original/low gets
+    frequency/factor, between them the two are blended linearly in
+    original/wavelength."""
+    import math
+
+    out = []
+    for i in range(dims // 2):
+        f = float(base) ** (-2.0 * i / dims)
+        if scaling:
+            factor, low, high, orig = (float(scaling[k])
+                                       for k in ("factor", "low", "high", "original"))
+            wavelen = 2.0 * math.pi / f
+            if wavelen > orig / low:
+                f = f / factor
+            elif wavelen >= orig / high:
+                smooth = (orig / wavelen - low) / (high - low)
+                f = (1.0 - smooth) * f / factor + smooth * f
+        out.append(f)
+    return torch.tensor(out, dtype=torch.float32)
+
+
+def attn_rope_prepare(qkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: torch.Tensor,
+                      inv_freq: torch.Tensor, H: int, G: int, D: int, Dv: int, eps: float,
+                      k_cache: torch.Tensor, v_cache: torch.Tensor, sb: SeqBatch) -> torch.Tensor:
+    """qkv [T, >= H*D + G*D + G*Dv] (q | k | v columns). RMS norm of every
+    query and key head over its D channels with the float32 weights [D]
+    (shared by heads), then rotation of the channel pairs (2i, 2i+1),
+    i < len(inv_freq), by position * inv_freq[i] — all in float32; k and v
+    are written to their pages; returns q [T, H, D]."""
+    T = qkv.shape[0]
+    assert 2 * inv_freq.numel() <= D
+    if not qkv.is_cuda:
+        pos = torch.tensor([sb.past[b] + i for b in range(sb.num_seqs)
+                            for i in range(sb.cu[b + 1] - sb.cu[b])], dtype=torch.float32)
+        return torch_ref.attn_rope_prepare(qkv, q_norm_w, k_norm_w, inv_freq, H, G, D, Dv, eps,
+                                           k_cache, v_cache, pos, sb.slot_mapping)
+    lib, hip = _lib()
+    assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype
+    assert k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, Dv)
+    for t in (q_norm_w, k_norm_w, inv_freq):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    assert q_norm_w.numel() == D and k_norm_w.numel() == D
+    q = torch.empty(T, H, D, dtype=qkv.dtype, device=qkv.device)
+    rc = lib.oa_attn_rope_prepare(
+        hip.current_stream_ptr(), qkv.data_ptr(), _rows(qkv), q_norm_w.data_ptr(),
+        k_norm_w.data_ptr(), inv_freq.data_ptr(), inv_freq.numel(), q.data_ptr(),
+        k_cache.data_ptr(), v_cache.data_ptr(), sb.slot_mapping.data_ptr(),
+        sb.seq_of_t.data_ptr(), sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.num_seqs, T,
+        H, G, D, Dv, eps, _dt(qkv))
+    hip.check(rc, "oa_attn_rope_prepare")
+    return q
+
+
+ACTS = {"silu": 0, "gelu_tanh": 1}
+
+
+def act_mul_rows(gu: torch.Tensor, inter: int, act: str = "silu") -> torch.Tensor:
+    """act(gu[:, :I]) * gu[:, I:] for a contiguous [M, 2I] buffer; act is
+    "silu" or "gelu_tanh" (the tanh form of gelu), evaluated in float32."""
+    if not gu.is_cuda:
+        g, u = gu.split([inter, inter], dim=-1)
+        return torch_ref.act_mul(g, u, act)
+    lib, hip = _lib()
+    assert gu.is_contiguous() and gu.shape[-1] == 2 * inter
+    M = gu.numel() // (2 * inter)
+    out = torch.empty(*gu.shape[:-1], inter, dtype=gu.dtype, device=gu.device)
+    hip.check(lib.oa_act_mul_rows(hip.current_stream_ptr(), gu.data_ptr(), out.data_ptr(),
+                                  M, inter, _dt(gu), ACTS[act]), "oa_act_mul_rows")
+    return out
+
+
+def route_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int,
+               groups: int = 1, keep: int = 1, scale: float = 1.0,
+               score: str = "sigmoid") -> Tuple[torch.Tensor, torch.Tensor]:
+    """Expert choice from float32 router logits [T, E]: returns (experts
+    int32 [T, top], weights float32 [T, top]). score "sigmoid" | "softmax";
+    c = score + correction (float32 [E], optional) ranks the experts; with
+    groups > 1 the experts are cut into `groups` runs of E/groups neighbours,
+    each run is rated max1(c) + max2(c), and only the `keep` top-rated runs
+    may be picked from. Weights: w_j = scale * s_j / (sum_k s_k + 1e-20) over
+    the picked experts' uncorrected scores s."""
+    T, E = logits.shape
+    assert logits.dtype == torch.float32 and E % max(groups, 1) == 0 and top <= E
+    if groups > 1:
+        assert keep * (E // groups) >= top, "too few eligible experts"
+    if not logits.is_cuda:
+        return torch_ref.route_topk(logits, correction, top, groups, keep, scale, score)
+    lib, hip = _lib()
+    logits = logits.contiguous()
+    idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    w = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    assert correction is None or (correction.dtype == torch.float32 and correction.is_contiguous())
+    rc = lib.oa_route_topk(
+        hip.current_stream_ptr(), logits.data_ptr(),
+        correction.data_ptr() if correction is not None else None, idx.data_ptr(),
+        w.data_ptr(), T, E, top, max(groups, 1), keep, float(scale),
+        0 if score == "sigmoid" else 1)
+    hip.check(rc, "oa_route_topk")
+    return idx, w
+
+
+def moe_pairs_mlp(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, idx: torch.Tensor,
+                  wts: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    """Routed experts for few tokens, two launches, no host sync and no
+    atomics: out[t] = sum_j wts[t,j] * W2[e_tj] (act(Wg[e_tj] x_t) * (Wu[e_tj] x_t)).
+    x [T, K]; w13 [E, 2I, K] (gate rows, then up rows); w2 [E, C, I]; idx
+    int32 [T, top]; wts float32 [T, top]. Any sizes, bf16 or float32. A
+    token's result does not depend on the other tokens of the batch."""
+    T, K = x.shape
+    E, I2, _ = w13.shape
+    I, C, top = I2 // 2, w2.shape[1], idx.shape[1]
+    if not x.is_cuda:
+        return torch_ref.moe_pairs_mlp(x, w13, w2, idx, wts, act)
+    lib, hip = _lib()
+    assert x.is_contiguous() and w13.is_contiguous() and w2.is_contiguous()
+    assert idx.is_contiguous() and idx.dtype == torch.int32
+    assert wts.is_contiguous() and wts.dtype == torch.float32
+    assert w13.dtype == x.dtype and w2.dtype == x.dtype and w2.shape == (E, C, I)
+    mid = torch.empty(T * top, I, dtype=x.dtype, device=x.device)
+    out = torch.empty(T, C, dtype=x.dtype, device=x.device)
+    hip.check(lib.oa_moe_pairs_gateup(
+        hip.current_stream_ptr(), x.data_ptr(), w13.data_ptr(), idx.data_ptr(), mid.data_ptr(),
+        T, top, E, I, K, _dt(x), ACTS[act]), "oa_moe_pairs_gateup")
+    hip.check(lib.oa_moe_pairs_down(
+        hip.current_stream_ptr(), mid.data_ptr(), w2.data_ptr(), idx.data_ptr(), wts.data_ptr(),
+        out.data_ptr(), T, top, E, C, I, _dt(x)), "oa_moe_pairs_down")
     return out
 
 

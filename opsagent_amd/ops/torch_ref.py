@@ -332,3 +332,146 @@ def gated_head_rms_norm(o, w, gate_logits, eps, out_dtype):
 
 def softcap(logits, cap):
     return cap * torch.tanh(logits.float() / cap)
+
+
+# ---------------------------------------------------------------------------
+# Blocks of sandwich-norm decoders with rotary window attention and routed
+# experts (same flat multi-sequence layout as above).
+
+
+def dyt_norm(y, post, residual, nxt, out_dtype):
+    """Dynamic-tanh norm dyt(x; w, b, a) = tanh(a x) w + b in float32.
+    With y and post = (w, b, a): residual += dyt(y; post), in place. With
+    nxt = (w, b, a): also returns dyt(residual; nxt) in out_dtype."""
+    if y is not None:
+        w, b, a = post
+        residual += torch.tanh(a.float() * y.float()) * w.float() + b.float()
+    if nxt is None:
+        return None
+    w, b, a = nxt
+    return (torch.tanh(a.float() * residual.float()) * w.float() + b.float()).to(out_dtype)
+
+
+def attn_rope_prepare(qkv, q_norm_w, k_norm_w, inv_freq, H, G, D, Dv, eps, k_cache, v_cache,
+                      positions, slot_mapping):
+    """Per-head RMS norm of q and k (weight [D] shared by heads), then rotation
+    of channel pairs (2i, 2i+1), i < len(inv_freq), by position * inv_freq[i];
+    k and v go to their cache slots, q is returned [T, H, D]."""
+    T = qkv.shape[0]
+    x = qkv[:, : H * D + G * D + G * Dv].float()
+    q = x[:, : H * D].reshape(T, H, D)
+    k = x[:, H * D : H * D + G * D].reshape(T, G, D)
+    v = x[:, H * D + G * D :].reshape(T, G, Dv)
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm_w.float()
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm_w.float()
+    r = 2 * inv_freq.numel()
+    if r:
+        ang = positions.float()[:, None] * inv_freq.float()[None, :]
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+
+        def rot(t):
+            a, b = t[..., 0:r:2], t[..., 1:r:2]
+            out = t.clone()
+            out[..., 0:r:2] = a * c - b * s
+            out[..., 1:r:2] = b * c + a * s
+            return out
+
+        q, k = rot(q), rot(k)
+    nb, bs = k_cache.shape[0], k_cache.shape[1]
+    sm = slot_mapping.long()
+    k_cache.view(nb * bs, G, D)[sm] = k.to(k_cache.dtype)
+    v_cache.view(nb * bs, G, Dv)[sm] = v.to(v_cache.dtype)
+    return q.to(qkv.dtype)
+
+
+def attention_paged(q, k_cache, v_cache, cu, past, block_table, scale, slopes=None,
+                    gate_logits=None, window=None, sinks=None):
+    """Causal softmax attention of each new token over its sequence's cached
+    keys. Options: a linear distance penalty slope_h*(i-j), a window (key j
+    seen iff i - j < window), a per-head sink term exp(sink_h) in the
+    denominator, a sigmoid gate on each head's output."""
+    T, H, D = q.shape
+    nb, bs, G, Dv = v_cache.shape
+    out = torch.empty(T, H, Dv, dtype=q.dtype, device=q.device)
+    rep = H // G
+    for b in range(len(cu) - 1):
+        lo, hi = cu[b], cu[b + 1]
+        if hi == lo:
+            continue
+        total = past[b] + hi - lo
+        first = max(0, past[b] - window + 1) if window else 0
+        fb = first // bs
+        first = fb * bs
+        nblk = (total + bs - 1) // bs
+        blocks = block_table[b, fb:nblk].long()
+        kk = k_cache[blocks].reshape(-1, G, D)[: total - first].float()
+        vv = v_cache[blocks].reshape(-1, G, Dv)[: total - first].float()
+        kk = kk.repeat_interleave(rep, dim=1)
+        vv = vv.repeat_interleave(rep, dim=1)
+        qs = q[lo:hi].float()
+        s = torch.einsum("ihd,jhd->hij", qs, kk) * scale
+        i = torch.arange(past[b], total, dtype=torch.float32).view(1, -1, 1)
+        j = torch.arange(first, total, dtype=torch.float32).view(1, 1, -1)
+        if slopes is not None:
+            s = s - slopes.float().view(H, 1, 1) * (i - j)
+        hide = j > i
+        if window:
+            hide = hide | (i - j >= window)
+        s = s.masked_fill(hide, float("-inf"))
+        if sinks is not None:
+            s = torch.cat([s, sinks.float().view(H, 1, 1).expand(H, s.shape[1], 1)], -1)
+        p = torch.softmax(s, dim=-1)
+        if sinks is not None:
+            p = p[..., :-1]
+        o = torch.einsum("hij,jhd->ihd", p, vv)
+        if gate_logits is not None:
+            o = o * torch.sigmoid(gate_logits[lo:hi].float()).unsqueeze(-1)
+        out[lo:hi] = o.to(q.dtype)
+    return out.view(T, H * Dv)
+
+
+def gelu_tanh(z):
+    return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+
+
+def act_mul(gate, up, act):
+    g = gate.float()
+    a = torch.nn.functional.silu(g) if act == "silu" else gelu_tanh(g)
+    return (a * up.float()).to(gate.dtype)
+
+
+def route_topk(logits, correction, top, groups, keep, scale, score):
+    """logits float32 [T, E] -> (experts int32 [T, top], weights float32
+    [T, top]). Scores are sigmoid or softmax of the logits; the choice uses
+    c = score + correction inside the `keep` top-rated of `groups` runs of
+    neighbouring experts (rating: max1(c) + max2(c)); weights
+    w_j = scale * s_j / (sum_k s_k + 1e-20) over the picked experts."""
+    T, E = logits.shape
+    s = torch.sigmoid(logits) if score == "sigmoid" else torch.softmax(logits, -1)
+    choice = s + correction.float() if correction is not None else s.clone()
+    if groups > 1:
+        per = E // groups
+        gs = choice.view(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+        best = gs.topk(keep, dim=-1).indices
+        ok = torch.zeros(T, groups, dtype=torch.bool, device=logits.device)
+        ok.scatter_(1, best, True)
+        choice = choice.masked_fill(~ok.repeat_interleave(per, dim=1), float("-inf"))
+    idx = choice.topk(top, dim=-1).indices
+    w = s.gather(1, idx)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+    return idx.to(torch.int32), w
+
+
+def moe_pairs_mlp(x, w13, w2, idx, wts, act):
+    """out[t] = sum_j wts[t, j] * W2[e] (act(Wg[e] x_t) * (Wu[e] x_t)), e =
+    idx[t, j]; w13 [E, 2I, K] holds gate rows then up rows, w2 [E, C, I]."""
+    T, top = idx.shape
+    inter = w13.shape[1] // 2
+    out = torch.zeros(T, w2.shape[1], dtype=torch.float32, device=x.device)
+    for t in range(T):
+        for j in range(top):
+            e = int(idx[t, j])
+            gu = torch.nn.functional.linear(x[t : t + 1], w13[e])
+            a = act_mul(gu[:, :inter], gu[:, inter:], act)
+            out[t] += wts[t, j] * torch.nn.functional.linear(a, w2[e])[0].float()
+    return out.to(x.dtype)
