@@ -29,7 +29,7 @@ SOURCES = [
 
 # the sequence-mixer kernels of hybrid decoders live in a library of their
 # own: a checkout that serves only such a model compiles just what it loads
-MIXER_SOURCES = ["mixers.hip"]
+MIXER_SOURCES = ["mixers.hip", "blocks.hip"]
 MIXER_OUT = os.path.join(
     os.path.dirname(os.path.abspath(__file__)), "libopsagent_mixers.so"
 )
@@ -59,6 +59,7 @@ def needs_rebuild(out: str = OUT, sources=None) -> bool:
         return True
     deps = [os.path.join(CSRC, s) for s in (sources or SOURCES)]
     deps.append(os.path.join(CSRC, "common.h"))
+    deps.append(os.path.join(CSRC, "mixer_util.h"))
     return any(_mtime(d) > out_t for d in deps)
 
 

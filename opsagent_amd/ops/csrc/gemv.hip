@@ -121,6 +121,16 @@ __global__ __launch_bounds__(256) void gemv_kernel(
     }
 }
 
+// gate activation of the fused gate-up kernels: 0 = silu, 1 = gelu in its tanh
+// approximation, g/2 * (1 + tanh(k (g + 0.044715 g^3))), k = sqrt(2/pi)
+__device__ __forceinline__ float gate_act(float g, int act) {
+    if (act == 1) {
+        const float t = tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g));
+        return 0.5f * g * (1.0f + t);
+    }
+    return g / (1.0f + __expf(-g));
+}
+
 // Fused gate-up + SiLU GEMV for the MLP up-projection: the fused weight
 // holds gate rows [0, I) and up rows [I, 2I); each wave computes BOTH rows
 // r and I + r and writes act[m][r] = silu(gate) * up directly — the separate
@@ -131,7 +141,7 @@ __global__ __launch_bounds__(256) void gemv_gateup_kernel(
     const uint32_t* __restrict__ w,  // [2I, K/2] (gate; up)
     uint32_t* __restrict__ out,      // [M, I] bf16
     const uint32_t* __restrict__ wn, // [K/2] rmsnorm weight (NORM only)
-    int I, int k2, float eps) {
+    int I, int k2, float eps, int act) {
     const int lane = threadIdx.x & (WAVE - 1);
     const int wid = threadIdx.x / WAVE;
 
@@ -173,8 +183,8 @@ __global__ __launch_bounds__(256) void gemv_gateup_kernel(
             const float g = wave_reduce_sum(accg[m]);
             const float u = wave_reduce_sum(accu[m]);
             if (lane == 0) {
-                const float act = g / (1.0f + __expf(-g)) * u;
-                reinterpret_cast<uint16_t*>(out)[(size_t)m * I + row] = f32_to_bf16(act);
+                const float a = gate_act(g, act) * u;
+                reinterpret_cast<uint16_t*>(out)[(size_t)m * I + row] = f32_to_bf16(a);
             }
         }
     }
@@ -186,13 +196,13 @@ extern "C" int oa_gemv_bf16_mfma(void* stream, const void* x, const void* w,
                                  int M, int N, int K, float eps, int mode,
                                  int gateup);
 
-extern "C" int oa_gemv_gateup_ex(void* stream, const void* x, const void* w,
-                                 void* out, const void* wn, int M, int I, int K,
-                                 float eps, int norm) {
+static int gemv_gateup_impl(void* stream, const void* x, const void* w,
+                            void* out, const void* wn, int M, int I, int K,
+                            float eps, int norm, int act) {
     if (K % 8 != 0) return -100;
     if (gemv_bf16_use_mfma(M, K, 1))
         return oa_gemv_bf16_mfma(stream, x, w, out, wn, nullptr, M, 2 * I, K,
-                                 eps, norm ? 1 : 0, 1);
+                                 eps, norm ? 1 : 0, 1 + act);
     const int k2 = K / 2;
     const int grid = min(2048, CEIL_DIV(I, 4));
 #define LAUNCH_GU(MV)                                                          \
@@ -201,12 +211,12 @@ extern "C" int oa_gemv_gateup_ex(void* stream, const void* x, const void* w,
             hipLaunchKernelGGL((gemv_gateup_kernel<MV, true>), dim3(grid),     \
                                dim3(256), 0, (hipStream_t)stream,              \
                                (const uint32_t*)x, (const uint32_t*)w,         \
-                               (uint32_t*)out, (const uint32_t*)wn, I, k2, eps);\
+                               (uint32_t*)out, (const uint32_t*)wn, I, k2, eps, act);\
         else                                                                   \
             hipLaunchKernelGGL((gemv_gateup_kernel<MV, false>), dim3(grid),    \
                                dim3(256), 0, (hipStream_t)stream,              \
                                (const uint32_t*)x, (const uint32_t*)w,         \
-                               (uint32_t*)out, (const uint32_t*)wn, I, k2, eps);\
+                               (uint32_t*)out, (const uint32_t*)wn, I, k2, eps, act);\
     } while (0)
     switch (M) {
         case 1: LAUNCH_GU(1); break;
@@ -226,9 +236,22 @@ extern "C" int oa_gemv_gateup_ex(void* stream, const void* x, const void* w,
     return 0;
 }
 
+extern "C" int oa_gemv_gateup_ex(void* stream, const void* x, const void* w,
+                                 void* out, const void* wn, int M, int I, int K,
+                                 float eps, int norm) {
+    return gemv_gateup_impl(stream, x, w, out, wn, M, I, K, eps, norm, 0);
+}
+
 extern "C" int oa_gemv_gateup(void* stream, const void* x, const void* w,
                               void* out, int M, int I, int K) {
-    return oa_gemv_gateup_ex(stream, x, w, out, nullptr, M, I, K, 0.0f, 0);
+    return gemv_gateup_impl(stream, x, w, out, nullptr, M, I, K, 0.0f, 0, 0);
+}
+
+// act: 0 silu, 1 gelu (tanh form)
+extern "C" int oa_gemv_gateup_act(void* stream, const void* x, const void* w,
+                                  void* out, int M, int I, int K, int act) {
+    if (act < 0 || act > 1) return -105;
+    return gemv_gateup_impl(stream, x, w, out, nullptr, M, I, K, 0.0f, 0, act);
 }
 
 // mode: 0 plain, 1 norm-prologue, 2 residual-add epilogue, 3 both
@@ -356,7 +379,7 @@ __global__ __launch_bounds__(256, 1) void gemv_bf16_mfma_kernel(
     uint32_t* __restrict__ out,       // [M, N] bf16 (gateup: [M, I])
     const uint32_t* __restrict__ wn,  // [K/2] rmsnorm weight (NORM)
     const uint32_t* __restrict__ res, // [M, N] residual (ADDRES)
-    int M, int N, int K, float eps) {
+    int M, int N, int K, float eps, int act) {
     constexpr int PF = GATEUP ? 4 : 8;
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
@@ -466,7 +489,7 @@ __global__ __launch_bounds__(256, 1) void gemv_bf16_mfma_kernel(
         }
         float v;
         if (GATEUP) {
-            v = sg / (1.0f + __expf(-sg)) * su;
+            v = gate_act(sg, act) * su;
         } else {
             v = sg;
             if (ADDRES)
@@ -515,7 +538,8 @@ extern "C" int oa_gemv_bf16_mfma(void* stream, const void* x, const void* w,
     hipLaunchKernelGGL((gemv_bf16_mfma_kernel<NORMV, RESV, GUV>), grid, block, \
                        shmem, (hipStream_t)stream, (const uint32_t*)x,         \
                        (const uint32_t*)w, (uint32_t*)out,                     \
-                       (const uint32_t*)wn, (const uint32_t*)res, M, N, K, eps)
+                       (const uint32_t*)wn, (const uint32_t*)res, M, N, K, eps, \
+                       gateup > 1 ? gateup - 1 : 0)
     if (gateup) {
         if (mode & 1) LAUNCH_BMF(true, false, true);
         else LAUNCH_BMF(false, false, true);

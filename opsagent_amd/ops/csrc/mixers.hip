@@ -16,45 +16,7 @@
 //
 // All sizes are run-time values; nothing assumes a multiple of 64.
 
-#include "common.h"
-
-#include <algorithm>
-#include <cstdlib>
-
-typedef uint16_t bf16s;  // bf16 storage
-
-__device__ __forceinline__ float ldf(const float* p, int64_t i) { return p[i]; }
-__device__ __forceinline__ float ldf(const bf16s* p, int64_t i) { return bf16_to_f32(p[i]); }
-__device__ __forceinline__ void stf(float* p, int64_t i, float v) { p[i] = v; }
-__device__ __forceinline__ void stf(bf16s* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
-
-// 8 consecutive elements at once (16-byte aligned for bf16, 32 for float32)
-__device__ __forceinline__ void ld8(const float* p, int64_t i, float* o) {
-    const float4 a = *reinterpret_cast<const float4*>(p + i);
-    const float4 b = *reinterpret_cast<const float4*>(p + i + 4);
-    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
-    o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
-}
-__device__ __forceinline__ void ld8(const bf16s* p, int64_t i, float* o) {
-    const uint4 a = *reinterpret_cast<const uint4*>(p + i);
-    o[0] = bf16_lo(a.x); o[1] = bf16_hi(a.x); o[2] = bf16_lo(a.y); o[3] = bf16_hi(a.y);
-    o[4] = bf16_lo(a.z); o[5] = bf16_hi(a.z); o[6] = bf16_lo(a.w); o[7] = bf16_hi(a.w);
-}
-__device__ __forceinline__ void st8(float* p, int64_t i, const float* v) {
-    *reinterpret_cast<float4*>(p + i) = make_float4(v[0], v[1], v[2], v[3]);
-    *reinterpret_cast<float4*>(p + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
-}
-__device__ __forceinline__ void st8(bf16s* p, int64_t i, const float* v) {
-    uint4 a;
-    a.x = pack_bf16x2(v[0], v[1]); a.y = pack_bf16x2(v[2], v[3]);
-    a.z = pack_bf16x2(v[4], v[5]); a.w = pack_bf16x2(v[6], v[7]);
-    *reinterpret_cast<uint4*>(p + i) = a;
-}
-
-__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
-__device__ __forceinline__ float softplusf_(float z) {
-    return fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z)));
-}
+#include "mixer_util.h"
 
 // ---------------------------------------------------------------------------
 // Causal convolution over time, per channel, continued from carried inputs.
@@ -437,9 +399,17 @@ __global__ __launch_bounds__(256) void attn_prepare_vec_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Softmax attention with a linear distance penalty over the paged cache.
+// Softmax attention over the paged cache with optional parts, each switched
+// by its argument:
 //   score(i, j) = q_i . k_j * scale - slope_h * (i - j),  j <= i
-//   out_i,h = sigmoid(gate_i,h) * sum_j softmax_j(score) v_j
+//                 (slopes null: no distance penalty)
+//   window > 0: only keys j > i - window are visible (the last `window`
+//                 positions up to the query); key tiles that end before
+//                 that range are never visited
+//   sinks given: Z_i,h = sum_j exp(score(i, j)) + exp(sink_h): the sink
+//                 enlarges the normaliser only, contributes no value
+//                 vector, and `scale` is not applied to it
+//   out_i,h = (sigmoid(gate_i,h)) * sum_j softmax_j(score) v_j  (gate null: 1)
 // grid = (query tiles, kv heads, key splits). A tile is up to TQ
 // consecutive new tokens of ONE sequence with all R = H/G query heads of
 // the kv head: ROWS = TQ*R rows share every staged key/value tile. Each of
@@ -458,8 +428,8 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
     TC* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ cu, const int* __restrict__ past,
     const int* __restrict__ block_table, int max_blocks, int block_size,
-    const float* __restrict__ slopes, int B, int H, int G, int D, int Dv, int TQ,
-    int KT, int kstride, float scale, int nsplit, int RB) {
+    const float* __restrict__ slopes, const float* __restrict__ sinks, int B, int H, int G,
+    int D, int Dv, int TQ, int KT, int kstride, float scale, int nsplit, int RB, int window) {
     extern __shared__ float lds[];
     // a block takes up to RB of the H/G query heads of one kv head
     const int hgroups = (H / G + RB - 1) / RB;
@@ -504,7 +474,9 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
         for (int c = 0; c < ATT_MAXV; ++c) acc[i][c] = 0.0f;
     }
     const int nkt = last_pos / KT + 1;
-    for (int kt = split; kt < nkt; kt += nsplit) {
+    // the first key any query of the tile sees
+    const int kt_first = window > 0 ? max(0, p0 - window + 1) / KT : 0;
+    for (int kt = kt_first + split; kt < nkt; kt += nsplit) {
         const int k0 = kt * KT;
         const int nk = min(KT, last_pos + 1 - k0);
         __syncthreads();
@@ -526,10 +498,11 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
             const int r = wave + 4 * ri;
             if (r >= rows) break;
             const int pos = p0 + r / R;
-            if (k0 > pos) continue;
-            const float slope = slopes[h0 + r % R];
+            const int kmin = window > 0 ? pos - window + 1 : 0;   // first key seen
+            if (k0 > pos || k0 + nk <= kmin) continue;
+            const float slope = slopes ? slopes[h0 + r % R] : 0.0f;
             float s = -INFINITY;
-            if (lane < nk && k0 + lane <= pos) {
+            if (lane < nk && k0 + lane <= pos && k0 + lane >= kmin) {
                 const float* qr = Qs + r * D;
                 const TC* kr = Ks + lane * kstride;
                 float a = 0.0f;
@@ -564,8 +537,9 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
         if (r >= rows) break;
         const int tok = lo + t0 + r / R, h = h0 + r % R;
         if (nsplit == 1) {
-            const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h));
-            const float inv = gt / l[ri];
+            const float gt = gate ? sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) : 1.0f;
+            const float lt = sinks ? l[ri] + expf(sinks[h] - m[ri]) : l[ri];
+            const float inv = gt / lt;
 #pragma unroll
             for (int c = 0; c < ATT_MAXV; ++c) {
                 const int ch = lane + 64 * c;
@@ -621,8 +595,8 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     bf16s* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ cu, const int* __restrict__ past,
     const int* __restrict__ block_table, int max_blocks, int block_size,
-    const float* __restrict__ slopes, int B, int H, int G, int D, int Dv, int HB,
-    float scale, int nsplit) {
+    const float* __restrict__ slopes, const float* __restrict__ sinks, int B, int H, int G,
+    int D, int Dv, int HB, float scale, int nsplit, int window) {
     // NT: 16-token sub-tiles per wave. Every K and V fragment read from LDS
     // feeds NT MFMAs, and a staged tile serves NT times the query rows.
     extern __shared__ float lds[];
@@ -661,8 +635,10 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int* bt = block_table + (int64_t)b * max_blocks;
     // softmax in the exp2 domain: log2(e) folded into the scale and the slope
     const float LOG2E = 1.4426950408889634f;
-    const float slope = slopes[h] * LOG2E;
+    const float slope = slopes ? slopes[h] * LOG2E : 0.0f;
     const float scale2 = scale * LOG2E;
+    // window as a bound that no position reaches when there is none
+    const int wlim = window > 0 ? window : 0x7fffffff;
 
     s4_t qf[NT][QK32 ? 1 : MAXD];
     s8_t qf8[NT][QK32 ? MAXD / 2 : 1];
@@ -735,8 +711,10 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
                                        : make_uint4(0, 0, 0, 0);
         }
     };
-    if (split < nkt) fetch(split);
-    for (int kt = split; kt < nkt; kt += nsplit) {
+    // key tiles before the window of the block's first query are skipped
+    const int kt_first = window > 0 ? max(0, pb + tile * TQ - window + 1) / MF_KT : 0;
+    if (kt_first + split < nkt) fetch(kt_first + split);
+    for (int kt = kt_first + split; kt < nkt; kt += nsplit) {
         const int k0 = kt * MF_KT;
         __syncthreads();
 #pragma unroll
@@ -758,7 +736,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         }
         __syncthreads();
         if (kt + nsplit < nkt) fetch(kt + nsplit);
-        if (wave_ntok <= 0 || k0 > wave_last) continue;
+        if (wave_ntok <= 0 || k0 > wave_last || k0 + MF_KT - 1 <= pb + t0 - wlim) continue;
         // S^T tiles: keys k0 + 16*mt + 4*lg + r, token lc of sub-tile u
         f4_t sc[NT][4];
 #pragma unroll
@@ -798,13 +776,18 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
             const float base = slope * (float)(pos[u] - k0 - 4 * lg);
             float mloc = -INFINITY;
             // only tiles that reach past some token of the wave need the mask
-            const bool diag = k0 + MF_KT - 1 > pb + t0 + 16 * u;
+            // (past the diagonal, or short of the window of the sub-tile's last token)
+            const bool diag = k0 + MF_KT - 1 > pb + t0 + 16 * u ||
+                              k0 <= pb + t0 + 16 * u + 15 - wlim;
 #pragma unroll
             for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     float v = fmaf(sc[u][mt][r], scale2, kbias[mt][r] - base);
-                    if (diag) v = (k0 + 16 * mt + 4 * lg + r <= pos[u]) ? v : -INFINITY;
+                    if (diag) {
+                        const int key = k0 + 16 * mt + 4 * lg + r;
+                        v = (key <= pos[u] && key > pos[u] - wlim) ? v : -INFINITY;
+                    }
                     sc[u][mt][r] = v;
                     mloc = fmaxf(mloc, v);
                 }
@@ -863,7 +846,8 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         if (lc >= ntok[u]) continue;
         const int tok = lo + t0 + 16 * u + lc;
         if (nsplit == 1) {
-            const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) / l[u];
+            const float lt = sinks ? l[u] + __builtin_amdgcn_exp2f(sinks[h] * LOG2E - m[u]) : l[u];
+            const float gt = (gate ? sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) : 1.0f) / lt;
             bf16s* orow = out + ((int64_t)tok * H + h) * Dv + 4 * lg;
 #pragma unroll
             for (int dt = 0; dt < MAXDV; ++dt)
@@ -892,8 +876,8 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
 template <typename TC>
 __global__ __launch_bounds__(64) void attn_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    const TC* __restrict__ gate, int64_t gs, TC* __restrict__ out, int H, int Dv,
-    int nsplit) {
+    const TC* __restrict__ gate, int64_t gs, const float* __restrict__ sinks,
+    TC* __restrict__ out, int H, int Dv, int nsplit) {
     __shared__ float wsh[64];
     const int64_t row = blockIdx.x;  // tok * H + h
     const int tok = (int)(row / H), h = (int)(row % H);
@@ -908,7 +892,8 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
         lsum = lsum * ((mx == -INFINITY) ? 0.0f : expf(mx - gmx)) + wave_reduce_sum(ls * wgt);
         mx = gmx;
     }
-    const float gt = sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) / lsum;
+    if (sinks) lsum += expf(sinks[h] - mx);
+    const float gt = (gate ? sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) : 1.0f) / lsum;
     float acc[ATT_MAXV];
 #pragma unroll
     for (int c = 0; c < ATT_MAXV; ++c) acc[c] = 0.0f;
@@ -1221,9 +1206,6 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(const TC* __restrict__ 
 
 // ===========================================================================
 // C entry points. dt: 0 = bf16 activations/weights, 1 = float32.
-static inline int grid_for(int64_t total) {
-    return (int)std::max<int64_t>(1, std::min<int64_t>(4096, CEIL_DIV(total, 256)));
-}
 
 // x_dt: type of x (0 bf16, 1 f32); dt: type of w and out
 extern "C" int oa_causal_conv_seq(void* stream, const void* x, int64_t xs, int x_dt,
@@ -1415,8 +1397,8 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                              int64_t gs, const void* k_cache, const void* v_cache, void* out,
                              void* part_o, void* part_ml, const void* cu, const void* past,
                              const void* block_table, int max_blocks, int block_size,
-                             const void* slopes, int B, int H, int G, int D, int Dv, int HB,
-                             float scale, int nsplit) {
+                             const void* slopes, const void* sinks, int B, int H, int G, int D,
+                             int Dv, int HB, float scale, int nsplit, int window) {
     if (lds_bytes > 48 * 1024)
         (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV, QK32, NT>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -1424,7 +1406,8 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                        (const bf16s*)q, (const bf16s*)gate, gs, (const bf16s*)k_cache,
                        (const bf16s*)v_cache, (bf16s*)out, (float*)part_o, (float*)part_ml,
                        (const int*)cu, (const int*)past, (const int*)block_table, max_blocks,
-                       block_size, (const float*)slopes, B, H, G, D, Dv, HB, scale, nsplit);
+                       block_size, (const float*)slopes, (const float*)sinks, B, H, G, D, Dv, HB,
+                       scale, nsplit, window);
 }
 
 // ntiles = sum_b ceil(n_b / TQ) (host-computed). part_* may be null when nsplit == 1.
@@ -1432,9 +1415,11 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
                                   const void* k_cache, const void* v_cache, void* out,
                                   void* part_o, void* part_ml, const void* cu, const void* past,
                                   const void* block_table, int max_blocks, int block_size,
-                                  const void* slopes, int T, int B, int ntiles, int H, int G,
-                                  int D, int Dv, float scale, int nsplit, int dt, int max_chunk) {
+                                  const void* slopes, const void* sinks, int T, int B, int ntiles,
+                                  int H, int G, int D, int Dv, float scale, int nsplit, int dt,
+                                  int max_chunk, int window) {
     if (T <= 0 || ntiles <= 0) return 0;
+    if (window < 0) return -105;
     int TQ, KT, ks, lds_bytes;
     int rc = oa_attn_bias_geometry(H, G, D, Dv, dt, max_chunk, &TQ, &KT, &ks, &lds_bytes);
     if (rc) return rc;
@@ -1445,7 +1430,7 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
         dim3 grid(ntiles, G * (R / HB), nsplit);
 #define MF_ARGS                                                                                   \
     s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out, part_o, part_ml, cu, past, block_table, \
-        max_blocks, block_size, slopes, B, H, G, D, Dv, HB, scale, nsplit
+        max_blocks, block_size, slopes, sinks, B, H, G, D, Dv, HB, scale, nsplit, window
 #define MF(A, Bv)                                                               \
     do {                                                                        \
         if (D % 32 == 0) launch_attn_mfma<A, Bv, true, 1>(MF_ARGS);             \
@@ -1470,8 +1455,8 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
 #define AT_ARGS(TC)                                                                      \
     (const TC*)q, (const TC*)gate, gs, (const TC*)k_cache, (const TC*)v_cache, (TC*)out,  \
         (float*)part_o, (float*)part_ml, (const int*)cu, (const int*)past,                \
-        (const int*)block_table, max_blocks, block_size, (const float*)slopes, B, H, G, D, \
-        Dv, TQ, KT, ks, scale, nsplit, rb
+        (const int*)block_table, max_blocks, block_size, (const float*)slopes,            \
+        (const float*)sinks, B, H, G, D, Dv, TQ, KT, ks, scale, nsplit, rb, window
         if (dt == 1)
             hipLaunchKernelGGL((attn_bias_paged_kernel<float>), grid, blk, lds_bytes, s, AT_ARGS(float));
         else
@@ -1483,11 +1468,11 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
         if (dt == 1)
             hipLaunchKernelGGL((attn_combine_kernel<float>), dim3((unsigned)((int64_t)T * H)), dim3(64), 0, s,
                                (const float*)part_o, (const float*)part_ml, (const float*)gate, gs,
-                               (float*)out, H, Dv, nsplit);
+                               (const float*)sinks, (float*)out, H, Dv, nsplit);
         else
             hipLaunchKernelGGL((attn_combine_kernel<bf16s>), dim3((unsigned)((int64_t)T * H)), dim3(64), 0, s,
                                (const float*)part_o, (const float*)part_ml, (const bf16s*)gate, gs,
-                               (bf16s*)out, H, Dv, nsplit);
+                               (const float*)sinks, (bf16s*)out, H, Dv, nsplit);
         HIP_CHECK_LAUNCH();
     }
     return 0;

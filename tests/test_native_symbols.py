@@ -19,7 +19,7 @@ ENTRY_POINTS = [
     "oa_attention_prefill", "oa_attention_prefill_variant",
     "oa_fp8_gemv_scratch_init", "oa_fused_add_rmsnorm", "oa_gemm_fp8",
     "oa_gemv", "oa_gemv_bf16_mfma", "oa_gemv_ex", "oa_gemv_fp8",
-    "oa_gemv_fp8_ex", "oa_gemv_fp8_mfma", "oa_gemv_gateup",
+    "oa_gemv_fp8_ex", "oa_gemv_fp8_mfma", "oa_gemv_gateup", "oa_gemv_gateup_act",
     "oa_gemv_gateup_ex", "oa_gemv_gateup_fp8", "oa_gemv_rw4", "oa_kv_write",
     "oa_masked_argmax", "oa_masked_argmax_f32", "oa_moe_down", "oa_moe_down_emaj", "oa_moe_gateup",
     "oa_moe_gateup_emaj", "oa_quant_fp8", "oa_rmsnorm", "oa_rope",
@@ -57,5 +57,7 @@ def test_mixers_library_exports():
     lib = ctypes.CDLL(MIXERS_LIB)
     for s in ["oa_causal_conv_seq", "oa_group_rmsnorm", "oa_attn_prepare",
               "oa_attn_bias_geometry", "oa_attn_bias_paged", "oa_delta_rule_fused",
-              "oa_softcap", "oa_silu_mul_rows", "oa_embed_rows"]:
+              "oa_softcap", "oa_silu_mul_rows", "oa_embed_rows", "oa_dyt_norm",
+              "oa_attn_rope_prepare", "oa_act_mul_rows", "oa_route_topk",
+              "oa_moe_pairs_gateup", "oa_moe_pairs_down"]:
         assert hasattr(lib, s), f"missing {s}"
