@@ -248,7 +248,8 @@ class LLMEngine:
         if self.hybrid:
             from opsagent_amd.engine.hybrid import HybridForCausalLM
 
-            # stateful mixers: no speculative rollback, no key-only prefix reuse
+            # recurrent state cannot roll back: no speculative decoding (prefix
+            # reuse is decided below, once the model's state shapes are known)
             self.spec_decode = False
             self.use_hipgraph = self.use_hipgraph and bool(cfg.get("hybrid_hipgraph", True))
             self.model = HybridForCausalLM(self.spec, self.dtype, self.device, self.seed)
@@ -297,10 +298,12 @@ class LLMEngine:
         if self.hybrid:
             # per-layer cache geometry comes from the model's mixers; every
             # live sequence also owns one slot of recurrent/convolution state
+            # keys alone restart a sequence only if no layer carries state
+            stateless = not any(self.model.state_layer_shapes())
             self.kv = PagedKVCache(
                 self.spec.num_layers, 0, 0, self.block_size, num_blocks, self.device,
                 self.dtype, layer_shapes=self.model.kv_layer_shapes(),
-                prefix_caching=False,
+                prefix_caching=stateless and bool(cfg.get("prefix_caching", True)),
             )
             self.state_pool = StateSlotPool(
                 int(cfg.get("state_slots", self.max_batch)),
@@ -775,6 +778,7 @@ class LLMEngine:
         for req, start, count in work:
             off += count
             req.prefill_done = min(len(req.prompt_ids), req.seq.num_cached)
+            req.seq.publish_full_blocks()      # no-op unless the cache reuses prefixes
             if req.seq.num_cached == len(req.seq.token_ids):
                 rows.append(off - 1)
                 batch.append(req)
