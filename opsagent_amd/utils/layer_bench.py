@@ -16,7 +16,13 @@ from typing import Dict, List
 
 import torch
 
-from opsagent_amd.engine.config import ModelSpec, povazen_config_dict, povazen_spec_from_dict
+from opsagent_amd.engine.config import (
+    ModelSpec,
+    povazen_config_dict,
+    povazen_spec_from_dict,
+    vazilorn_config_dict,
+    vazilorn_spec_from_dict,
+)
 
 # (name, width, heads, kv_heads, head dim, ff, layers)
 SIZES = [
@@ -37,7 +43,36 @@ def specs_for(size) -> Dict[str, object]:
                             kv_heads=kv, dim=dim, vdim=dim, ff=ff, delta_heads=heads),
         name=f"povazen-{name}",
     )
-    return {"llama": llama, "povazen": hybrid}
+    # routed feed-forwards of equal shape in both families: 16 experts of
+    # ff/8, 4 per token, one shared expert of the same size
+    experts, top, eff = 16, 4, ff // 8
+    llama_moe = dataclasses.replace(
+        llama, name=f"llama-moe-{name}", moe_num_experts=experts, moe_top_k=top,
+        moe_intermediate_size=eff, moe_shared_experts=1,
+    )
+
+    def vz(pattern, window, tag):
+        return vazilorn_spec_from_dict(
+            vazilorn_config_dict(vocab=32000, width=width, pattern=pattern * layers, heads=heads,
+                                 kv_heads=kv, dim=dim, vdim=dim, ff=ff, window=window,
+                                 experts=experts, top=top, expert_ff=eff, groups=4, keep=2,
+                                 router_scale=2.0, shared_ff=eff, rot_base=500000.0),
+            name=f"vazilorn-{tag}-{name}",
+        )
+
+    return {
+        "llama": llama, "povazen": hybrid, "llama-moe": llama_moe,
+        # a window wider than the prompt: the attention kernels do llama's work
+        "vazilorn": vz("d", 8192, "dense"),
+        # a window that pays: keys beyond it are never read
+        "vazilorn-w512": vz("d", 512, "w512"),
+        "vazilorn-moe": vz("m", 8192, "moe"),
+    }
+
+
+# which model each one is measured against
+BASELINE_OF = {"povazen": "llama", "vazilorn": "llama", "vazilorn-w512": "llama",
+               "vazilorn-moe": "llama-moe"}
 
 
 def _run(spec, batch: int, prompt: int, decode: int, reps: int) -> Dict[str, float]:
@@ -89,10 +124,11 @@ def run(sizes=None, prompt: int = 2048, decode: int = 64, batches=(1, 8), reps: 
             for m in models:
                 r = _run(specs[m], b, prompt, decode, reps)
                 row[m] = {k: round(v, 2) for k, v in r.items()}
-            if "llama" in row and "povazen" in row:
-                row["povazen_vs_llama"] = {
-                    "prefill": round(row["povazen"]["prefill_tok_s"] / row["llama"]["prefill_tok_s"], 3),
-                    "decode": round(row["povazen"]["decode_tok_s"] / row["llama"]["decode_tok_s"], 3),
-                }
+            for m, base in BASELINE_OF.items():
+                if m in row and base in row:
+                    row[f"{m}_vs_{base}".replace("-", "_")] = {
+                        "prefill": round(row[m]["prefill_tok_s"] / row[base]["prefill_tok_s"], 3),
+                        "decode": round(row[m]["decode_tok_s"] / row[base]["decode_tok_s"], 3),
+                    }
             rows.append(row)
     return rows
